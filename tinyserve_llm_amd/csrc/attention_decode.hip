@@ -50,7 +50,7 @@ attn_decode_mfma_kernel(bf16_t* __restrict__ out, float* __restrict__ part_o, fl
   int pos = positions[t];
   int seq = seq_of_token[t];                    // (asked for with the position: one trip to memory, not one after the other;
   asm volatile("" : "+s"(pos), "+s"(seq));      //  left to itself the compiler fetches it when it has seen that the chunk is visible)
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = ts_first_key(pos, window);
   const int k0 = split * chunk;
   if (k0 > pos || k0 + chunk <= lo) return;     // nothing of this chunk is visible
   const int32_t* table = block_tables + (int64_t)seq * max_blocks;
@@ -155,7 +155,7 @@ attn_decode_combine_kernel(bf16_t* __restrict__ out, const float* __restrict__ p
   const int t = blockIdx.x / nh, lane = threadIdx.x;
   const int64_t th = blockIdx.x;
   const int pos = positions[t];
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = ts_first_key(pos, window);
   const int s0 = min(lo / chunk, num_splits - 1), s1 = min(pos / chunk, num_splits - 1);  // the last chunk is open-ended
   const float* ml = part_ml + th * num_splits * 2;
   float M = -INFINITY;

@@ -3,7 +3,7 @@
 //   * `ts_qkv_finish`: what lies between the q|k|v projection and the cache. Rotary positions on the first
 //     `rot` dimensions of each q and k head, pairing (2i, 2i+1) (interleaved) or (i, i + rot/2) (halves), the
 //     angle p * f_i taken in 64-bit from a table of frequencies (no table over positions: a request may be of
-//     any length); then, optionally, each q and k head divided by its root mean square, and each value head
+//     any length), cosine and sine times `amplitude` (1 for plain rotary positions); then, optionally, each q and k head divided by its root mean square, and each value head
 //     likewise; q goes to [tokens, heads, dim], k and v to their cache slots. Key and value heads may
 //     differ in size.
 //   * `ts_paged_attention_general`: one wavefront per (token, query head) over the request's pages, causal,
@@ -27,7 +27,7 @@ qkv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restri
                   const double* __restrict__ freqs, const int32_t* __restrict__ positions,
                   const int32_t* __restrict__ slots, int num_tokens, int nh, int nkv, int hd, int vd_size, int rot,
                   int interleaved, int qk_norm, float qk_eps, int v_norm, float v_eps, int page_size, int64_t kp,
-                  int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int with_values) {
+                  int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int with_values, float amplitude) {
   __shared__ float head_s[AG_WAVES][AG_MAX_HD];
   __shared__ float cos_s[AG_MAX_HD / 2], sin_s[AG_MAX_HD / 2];
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
@@ -42,8 +42,8 @@ qkv_finish_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* __restri
     const float a = (float)fma(-turns, 6.283185307179586, angle);
     float sn, cs;
     sincosf(a, &sn, &cs);
-    cos_s[pair] = cs;
-    sin_s[pair] = sn;
+    cos_s[pair] = cs * amplitude;
+    sin_s[pair] = sn * amplitude;
   }
   __syncthreads();
   const int64_t row = (int64_t)(nh + nkv) * hd + (int64_t)nkv * vd_size;
@@ -132,7 +132,7 @@ qkv_finish_pieces_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* _
                          const double* __restrict__ freqs, const int32_t* __restrict__ positions,
                          const int32_t* __restrict__ slots, int num_tokens, int nh, int nkv, int hd, int vd_size, int rot,
                          int interleaved, int qk_norm, float qk_eps, int v_norm, float v_eps, int page_size, int64_t kp,
-                         int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int with_values, int slices) {
+                         int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh, int64_t vd, int with_values, float amplitude, int slices) {
   const int64_t gid = (int64_t)blockIdx.x * (AG_WAVES * TS_WAVE) + threadIdx.x;
   const int piece = (int)(gid % GS);
   const int slice = (int)((gid / GS) % slices);
@@ -158,6 +158,7 @@ qkv_finish_pieces_kernel(TO* __restrict__ q_out, TO* __restrict__ k_cache, TO* _
         const double angle = (double)pos * freqs[pair];
         const double turns = rint(angle * 0.15915494309189535);
         sincosf((float)fma(-turns, 6.283185307179586, angle), &sn[e], &cs[e]);
+        cs[e] *= amplitude; sn[e] *= amplitude;
       }
       if (interleaved && (e & 1)) { cs[e] = cs[e - 1]; sn[e] = sn[e - 1]; }
     }
@@ -279,7 +280,7 @@ extern "C" int ts_qkv_finish(void* q_out, void* k_cache, void* v_cache, const vo
                              const int32_t* positions, const int32_t* slots, int num_tokens, int nh, int nkv, int hd,
                              int vd_size, int rot, int interleaved, int qk_norm, float qk_eps, int v_norm, float v_eps,
                              int page_size, int64_t kp, int64_t ks, int64_t kh, int64_t vp, int64_t vs, int64_t vh,
-                             int64_t vd, int in_dtype, int out_dtype, hipStream_t stream) {
+                             int64_t vd, int in_dtype, int out_dtype, float amplitude, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (hd <= 0 || hd > AG_MAX_HD || vd_size <= 0 || vd_size > AG_MAX_HD || nh <= 0 || nkv <= 0 || rot < 0 || rot > hd || rot % 2 ||
       page_size <= 0 || (rot > 0 && !freqs))
@@ -302,7 +303,7 @@ extern "C" int ts_qkv_finish(void* q_out, void* k_cache, void* v_cache, const vo
   const unsigned piece_blocks = (unsigned)((piece_threads + AG_WAVES * TS_WAVE - 1) / (AG_WAVES * TS_WAVE));
 #define QF_ARGS(TI, TO) \
       (TO*)q_out, (TO*)k_cache, (TO*)v_cache, (const TI*)qkv, freqs, positions, slots, num_tokens, nh, nkv, hd, vd_size, rot, \
-      interleaved, qk_norm, qk_eps, v_norm, v_eps, page_size, kp, ks, kh, vp, vs, vh, vd, !v_tiles
+      interleaved, qk_norm, qk_eps, v_norm, v_eps, page_size, kp, ks, kh, vp, vs, vh, vd, !v_tiles, amplitude
 #define QF_LAUNCH(TI, TO) \
   if (!pieces) qkv_finish_kernel<TI, TO><<<(unsigned)blocks, AG_WAVES * TS_WAVE, 0, stream>>>(QF_ARGS(TI, TO)); \
   else if (gs == 4) qkv_finish_pieces_kernel<TI, TO, 4><<<piece_blocks, AG_WAVES * TS_WAVE, 0, stream>>>(QF_ARGS(TI, TO), slices); \
@@ -343,7 +344,7 @@ paged_attention_general_kernel(T* __restrict__ out, const T* __restrict__ q, con
   for (int d = lane; d < hd; d += TS_WAVE) q_s[wave][d] = Num<T>::ld(qrow + d);
   wave_sync();
 
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = ts_first_key(pos, window);
   // the sink is a key of score 0 without a value: it starts the running maximum and the sum
   // (a learned sink is the same key with a score of its own)
   float m = sinks ? sinks[h] : sink ? 0.f : -INFINITY, l = (sinks || sink) ? 1.f : 0.f;

@@ -73,7 +73,7 @@ prefill_tile(PrefillLds<HD>& lds, int tile, int kvh, bf16_t* __restrict__ out, c
     tk[j] = (wave * RT + j) * tpt + r / G;
     const bool ok = r / G < tpt && tk[j] < ntok;
     pos[j] = ok ? positions[t0 + tk[j]] : -1;               // -1: no key is visible, the row stays empty
-    lo[j] = (window > 0 && pos[j] - window + 1 > 0) ? pos[j] - window + 1 : 0;
+    lo[j] = ts_first_key(pos[j], window);
     if (!ok) tk[j] = -1;
     pmax = max(pmax, pos[j]);
     lmin = min(lmin, ok ? lo[j] : 0x7fffffff);

@@ -54,7 +54,7 @@ paged_attention_wave_kernel(T* __restrict__ out, const T* __restrict__ q, const 
   for (int d = lane; d < hd; d += TS_WAVE) q_s[wave][d] = Num<T>::ld(qrow + d);
   wave_sync();
 
-  const int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  const int lo = ts_first_key(pos, window);
   float m = -INFINITY, l = 0.f;
   float acc[ATT_MAX_HD / TS_WAVE] = {0.f, 0.f, 0.f, 0.f};
 

@@ -55,6 +55,15 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
+// The first key that the query at position `pos` sees (it sees up to `pos`). `window` > 0: the last `window`
+// positions, itself included (a sliding window); `window` < 0: the positions of its own chunk of -window
+// positions, chunks counted from position 0 of the request; 0: every key before it.
+__device__ __forceinline__ int ts_first_key(int pos, int window) {
+  if (window > 0) return pos - window + 1 > 0 ? pos - window + 1 : 0;
+  if (window < 0) return pos - pos % (-window);
+  return 0;
+}
+
 // Orders shared-memory writes of a wavefront before the reads of its other lanes.
 __device__ __forceinline__ void wave_sync() {
   __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

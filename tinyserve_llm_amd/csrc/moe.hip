@@ -1,13 +1,15 @@
 // A mixture of experts: every token goes through `top` of `experts` small gated feed-forward layers.
 //   * `ts_moe_route`: router logits z = W_r h in 32-bit (h as it is stored), scores s = sigmoid(z); the `top`
 //     experts with the largest s + correction are chosen (ties: the lower index); their weights are their s,
-//     divided by the chosen ones' sum (+ 1e-20) if `normalize`, times `scale`.
+//     divided by the chosen ones' sum (+ 1e-20) if `normalize`, times `scale`. With `softmax_chosen` the logits
+//     themselves are the scores, and the weights are the softmax over the chosen experts' logits alone.
 //   * `ts_moe_group`: the step's (token, choice) pairs grouped by expert, and the groups cut into tiles of rows
 //     that one workgroup of the product takes: [expert, first index, rows] per tile, rows 0 for the tiles of the
 //     launch that the step does not fill (the launch is sized for the worst case, so nothing comes back to the host).
 //   * `ts_moe_gemm`: for every tile, rows of the operand (a token's row, or a pair's) times the tile's expert's
 //     matrix; with `glu` the matrix holds gate rows, then up rows, and the capped gated unit
 //     g = min(gate, L), u = clamp(up, -L, L), y = g sigmoid(slope g) (u + shift) leaves instead of the sums.
+//     Without `glu`, `act` 1 squares the sums' positive parts on their way out (experts of the form W_down relu(W_up h)^2).
 //     Every row's sums run over k in ascending order whatever the tile it lands in.
 //   * `ts_moe_combine`: out[token] = sum over its choices, in order, of weight * the pair's row (+ a shared
 //     expert's row).
@@ -26,7 +28,7 @@ template <typename TX>
 __global__ void __launch_bounds__(MOE_ROUTE_THREADS)
 moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const TX* __restrict__ x,
                  const float* __restrict__ router, const float* __restrict__ correction, int num_tokens, int K, int E, int top,
-                 float scale, int normalize) {
+                 float scale, int normalize, int softmax_chosen) {
   extern __shared__ float lds[];
   float* s_s = lds;                                       // [MOE_ROUTE_TOKENS][E] logits, then scores
   float* c_s = lds + MOE_ROUTE_TOKENS * E;                // [MOE_ROUTE_TOKENS][E] choice scores
@@ -87,7 +89,7 @@ moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const
   }
   __syncthreads();
   for (int i = threadIdx.x; i < MOE_ROUTE_TOKENS * E; i += MOE_ROUTE_THREADS) {
-    const float sc = 1.0f / (1.0f + expf(-s_s[i]));
+    const float sc = softmax_chosen ? s_s[i] : 1.0f / (1.0f + expf(-s_s[i]));
     s_s[i] = sc;
     c_s[i] = sc + (correction ? correction[i % E] : 0.f);
   }
@@ -116,8 +118,12 @@ moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const
     if (lane == 0) c_s[r * E + at] = -INFINITY;
     wave_sync();
   }
+  if (softmax_chosen) {                                   // the chosen logits' softmax: the first choice is the largest
+    const float top_logit = __shfl(my_pick, 0, TS_WAVE);
+    my_pick = lane < top ? expf(my_pick - top_logit) : 0.f;
+  }
   const float total = wave_sum(my_pick);                  // (the lanes beyond `top` hold 0)
-  const float mult = (normalize ? 1.0f / (total + 1e-20f) : 1.0f) * scale;
+  const float mult = (softmax_chosen ? 1.0f / total : normalize ? 1.0f / (total + 1e-20f) : 1.0f) * scale;
   if (lane < top) {
     ids_out[(int64_t)t * top + lane] = my_choice;
     w_out[(int64_t)t * top + lane] = my_pick * mult;
@@ -126,17 +132,17 @@ moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const
 
 extern "C" int ts_moe_route(int32_t* ids_out, float* w_out, const void* x, int x_dtype, const float* router,
                             const float* correction, int num_tokens, int K, int E, int top, float scale, int normalize,
-                            hipStream_t stream) {
+                            int softmax_chosen, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (K <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > MOE_MAX_TOP || top > E) return TS_BAD_SHAPE;
   const unsigned blocks = (num_tokens + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS;
   const size_t lds = (size_t)MOE_ROUTE_TOKENS * (2 * E + MOE_ROUTE_CHUNK) * sizeof(float);
   if (x_dtype == 0)
     moe_route_kernel<float><<<blocks, MOE_ROUTE_THREADS, lds, stream>>>(ids_out, w_out, (const float*)x, router, correction,
-                                                                        num_tokens, K, E, top, scale, normalize);
+                                                                        num_tokens, K, E, top, scale, normalize, softmax_chosen);
   else if (x_dtype == 1)
     moe_route_kernel<bf16_t><<<blocks, MOE_ROUTE_THREADS, lds, stream>>>(ids_out, w_out, (const bf16_t*)x, router, correction,
-                                                                         num_tokens, K, E, top, scale, normalize);
+                                                                         num_tokens, K, E, top, scale, normalize, softmax_chosen);
   else return TS_BAD_DTYPE;
   return ts_check_launch();
 }
@@ -203,6 +209,12 @@ extern "C" int ts_moe_group(const int32_t* ids, int32_t* sorted, int32_t* tiles,
 #define MOE_BN 64
 #define MOE_KC 32
 
+// What an ungated expert's sums pass on their way out: 0 nothing, 1 the square of relu.
+static __device__ __forceinline__ float moe_act(float s, int act) {
+  if (act == 1) { const float r = fmaxf(s, 0.f); return r * r; }
+  return s;
+}
+
 static __device__ __forceinline__ float moe_unit(float g, float u, float limit, float slope, float shift) {
   if (limit > 0.f) {
     g = fminf(g, limit);
@@ -215,7 +227,7 @@ static __device__ __forceinline__ float moe_unit(float g, float u, float limit, 
 template <typename TX, typename TO>
 __global__ void __launch_bounds__(MOE_THREADS)
 moe_gemm_kernel(TO* __restrict__ out, const TX* __restrict__ x, const TX* __restrict__ w, const int32_t* __restrict__ sorted,
-                const int32_t* __restrict__ tiles, int src_div, int N, int K, int glu, float limit, float slope, float shift) {
+                const int32_t* __restrict__ tiles, int src_div, int N, int K, int glu, float limit, float slope, float shift, int act) {
   __shared__ float x_s[MOE_BM][MOE_KC + 1];
   __shared__ float w_s[2][MOE_BN][MOE_KC + 1];
   __shared__ int row_s[MOE_BM];
@@ -261,7 +273,7 @@ moe_gemm_kernel(TO* __restrict__ out, const TX* __restrict__ x, const TX* __rest
   for (int r = 0; r < 4; ++r) {
     const int p = row_s[ty * 4 + r];
     if (p < 0) continue;
-    const float y = glu ? moe_unit(acc[r], acc2[r], limit, slope, shift) : acc[r];
+    const float y = glu ? moe_unit(acc[r], acc2[r], limit, slope, shift) : moe_act(acc[r], act);
     Num<TO>::st(out + (int64_t)p * N + n0 + tx, y);
   }
 }
@@ -301,7 +313,7 @@ template <int TM, int TN, bool GLU, typename TO>
 __global__ void __launch_bounds__(MOE_THREADS)
 moe_gemm_mfma_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                      const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles, int src_div, int N, int K,
-                     float limit, float slope, float shift) {
+                     float limit, float slope, float shift, int act) {
   constexpr int SETS = GLU ? 2 : 1;
   const int tile = blockIdx.x;
   const int rows = tiles[3 * tile + 2];
@@ -361,7 +373,7 @@ moe_gemm_mfma_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const b
 #pragma unroll
       for (int c = 0; c < 4; ++c) {
         if constexpr (GLU) y[c] = moe_unit(acc[0][j][i][c], acc[1][j][i][c], limit, slope, shift);
-        else y[c] = acc[0][j][i][c];
+        else y[c] = moe_act(acc[0][j][i][c], act);
       }
       moe_store4(orow + col, y, N - col);
     }
@@ -377,7 +389,7 @@ template <bool GLU, typename TO>
 __global__ void __launch_bounds__(MOE_THREADS)
 moe_gemm_stream_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                        const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles, int src_div, int N, int K,
-                       float limit, float slope, float shift) {
+                       float limit, float slope, float shift, int act) {
   constexpr int SETS = GLU ? 2 : 1;
   constexpr int WAVES = MOE_THREADS / TS_WAVE, DEPTH = 4;
   __shared__ moe_f32x4 part_s[WAVES - 1][SETS][TS_WAVE];
@@ -437,7 +449,7 @@ moe_gemm_stream_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const
 #pragma unroll
   for (int c = 0; c < 4; ++c) {
     if constexpr (GLU) y[c] = moe_unit(acc[0][c], acc[1][c], limit, slope, shift);
-    else y[c] = acc[0][c];
+    else y[c] = moe_act(acc[0][c], act);
   }
   moe_store4(orow + c0, y, N - c0);
 }
@@ -454,7 +466,7 @@ template <int WM, int WN, bool GLU, typename TO>
 __global__ void __launch_bounds__(WM * WN * TS_WAVE)
 moe_gemm_lds_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w,
                     const int32_t* __restrict__ sorted, const int32_t* __restrict__ tiles, int num_tiles, int col_blocks,
-                    int src_div, int N, int K, float limit, float slope, float shift) {
+                    int src_div, int N, int K, float limit, float slope, float shift, int act) {
   constexpr int BM = 128, BN = 128;
   constexpr int THREADS = WM * WN * TS_WAVE;
   constexpr int FX = BM / 16 * 2, FW = BN / 16 * 2;       // fragments (a kilobyte each) of a k-step of 64
@@ -589,7 +601,7 @@ moe_gemm_lds_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf
 #pragma unroll
       for (int j = 0; j < TN; ++j) {
         const int n = n0 + (wn * TN + j) * 16 + 4 * g;
-        const float y[4] = {acc[j][i][0], acc[j][i][1], acc[j][i][2], acc[j][i][3]};
+        const float y[4] = {moe_act(acc[j][i][0], act), moe_act(acc[j][i][1], act), moe_act(acc[j][i][2], act), moe_act(acc[j][i][3], act)};
         moe_store4(orow + n, y, N - n);
       }
     }
@@ -598,8 +610,9 @@ moe_gemm_lds_kernel(TO* __restrict__ out, const bf16_t* __restrict__ x, const bf
 
 extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype, const void* w, const int32_t* sorted,
                            const int32_t* tiles, int max_tiles, int tile_rows, int src_div, int N, int K, int glu, float limit,
-                           float slope, float shift, hipStream_t stream) {
+                           float slope, float shift, int act, hipStream_t stream) {
   if (max_tiles <= 0) return TS_OK;
+  if (act < 0 || act > 1 || (glu && act)) return TS_BAD_SHAPE;
   if (N <= 0 || K <= 0 || src_div <= 0 || (tile_rows != 16 && tile_rows != 64 && tile_rows != 128)) return TS_BAD_SHAPE;
   const bool mfma = x_dtype == 1 && K % 32 == 0 && (((uintptr_t)x | (uintptr_t)w) & 15) == 0;
   if (tile_rows == 128) {
@@ -610,7 +623,7 @@ extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype,
     const unsigned grid = (unsigned)((items + MOE_DIES - 1) / MOE_DIES * MOE_DIES);
 #define MOE_LDS(WM, WN, GLU, TO) \
     moe_gemm_lds_kernel<WM, WN, GLU, TO><<<grid, WM * WN * TS_WAVE, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w, sorted, \
-                                                                                  tiles, max_tiles, col_blocks, src_div, N, K, limit, slope, shift)
+                                                                                  tiles, max_tiles, col_blocks, src_div, N, K, limit, slope, shift, act)
     if (glu && out_dtype == 1) MOE_LDS(4, 1, true, bf16_t);
     else if (!glu && out_dtype == 0) MOE_LDS(2, 2, false, float);
     else if (!glu && out_dtype == 1) MOE_LDS(2, 2, false, bf16_t);
@@ -624,7 +637,7 @@ extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype,
       if (grid.y > 65535) return TS_BAD_SHAPE;
 #define MOE_STREAM(GLU, TO) \
       moe_gemm_stream_kernel<GLU, TO><<<grid, MOE_THREADS, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w, sorted, tiles, \
-                                                                        src_div, N, K, limit, slope, shift)
+                                                                        src_div, N, K, limit, slope, shift, act)
       if (glu && out_dtype == 1) MOE_STREAM(true, bf16_t);
       else if (!glu && out_dtype == 0) MOE_STREAM(false, float);
       else if (!glu && out_dtype == 1) MOE_STREAM(false, bf16_t);
@@ -637,7 +650,7 @@ extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype,
     if (grid.y > 65535) return TS_BAD_SHAPE;
 #define MOE_MFMA(TM, GLU, TO) \
     moe_gemm_mfma_kernel<TM, 2, GLU, TO><<<grid, MOE_THREADS, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w, sorted, \
-                                                                           tiles, src_div, N, K, limit, slope, shift)
+                                                                           tiles, src_div, N, K, limit, slope, shift, act)
     if (glu && out_dtype == 1) MOE_MFMA(4, true, bf16_t);
     else if (!glu && out_dtype == 0) MOE_MFMA(4, false, float);
     else if (!glu && out_dtype == 1) MOE_MFMA(4, false, bf16_t);
@@ -650,7 +663,7 @@ extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype,
   if (grid.y > 65535) return TS_BAD_SHAPE;
 #define MOE_LAUNCH(TX, TO) \
   moe_gemm_kernel<TX, TO><<<grid, MOE_THREADS, 0, stream>>>((TO*)out, (const TX*)x, (const TX*)w, sorted, tiles, src_div, N, K, \
-                                                            glu, limit, slope, shift)
+                                                            glu, limit, slope, shift, act)
   if (x_dtype == 0 && out_dtype == 0) MOE_LAUNCH(float, float);
   else if (x_dtype == 1 && out_dtype == 1) MOE_LAUNCH(bf16_t, bf16_t);
   else if (x_dtype == 1 && out_dtype == 0) MOE_LAUNCH(bf16_t, float);

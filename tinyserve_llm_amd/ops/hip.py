@@ -83,7 +83,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_bias_activation": [p, i, p, i, p, i, i, i, i, p],
         "ts_mingru_scan": [p, i, p, i, p, i, p, p, p, i, i, i, p],
         "ts_mingru_scan_chunks": [p, i, p, i, p, i, p, p, p, p, p, i, i, i, p],
-        "ts_qkv_finish": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, f, i, f, i, i64, i64, i64, i64, i64, i64, i64, i, i, p],
+        "ts_qkv_finish": [p, p, p, p, p, p, p, i, i, i, i, i, i, i, i, f, i, f, i, i64, i64, i64, i64, i64, i64, i64, i, i, f, p],
         "ts_paged_attention_general": [p, p, p, p, p, p, p, i, i, i, i, i, i, i64, i64, i64, i64, i64, i64, i64, i, f, f, i, i,
                                        i, i, p, p, p, i64, p],
         "ts_dyt": [p, i, p, i, p, i, p, i, p, p, p, p, i, i, p],
@@ -93,9 +93,16 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_conv_finish": [p, p, p, p, i64, p, p, p, p, f, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i64, i64, i64, i64, i64,
                            i64, i64, i, i, i, p],
         "ts_conv_state_update": [p, p, i64, p, p, i, i, i, i, p],
-        "ts_moe_route": [p, p, p, i, p, p, i, i, i, i, f, i, p],
+        "ts_moe_route": [p, p, p, i, p, p, i, i, i, i, f, i, i, p],
         "ts_moe_group": [p, p, p, i, i, i, i, p],
-        "ts_moe_gemm": [p, i, p, i, p, p, p, i, i, i, i, i, i, f, f, f, p],
+        "ts_moe_gemm": [p, i, p, i, p, p, p, i, i, i, i, i, i, f, f, f, i, p],
+        "ts_segment_rmsnorm": [p, i, i64, p, i64, i, p, f, i, p],
+        "ts_latent_finish": [p, p, i, p, i64, i, i, i, i, i, p, p, f, p, f, p, p, i, i64, i64, i, p],
+        "ts_rotate_heads": [p, i, i64, i64, p, i64, i64, i, i, i, p, f, p, i, p],
+        "ts_heads_gemm": [p, i, i64, i64, p, i, i64, i64, p, i, i64, i64, i64, i, i, i, i, p, i64, p],
+        "ts_paged_attention_latent": [p, i, p, i, p, i, p, p, p, i, i, i, i, i, i64, i64, i, f, i, i, p],
+        "ts_mlstm_scan": [p, p, i64, p, p, p, p, p, i, i, i, i, i, f, f, p],
+        "ts_mlstm_finish": [p, i, p, p, p, i64, i, i, i, f, p],
         "ts_moe_combine": [p, p, p, p, i, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p, i, p],
@@ -716,7 +723,7 @@ def paged_attention_prefill(q: torch.Tensor, k_cache: torch.Tensor, v_cache: tor
 def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, ctx, space: int,
                     scale: float, window: int = 0, leave_split: bool = False, softcap: float = 0.0,
                     sink: bool = False, sinks: torch.Tensor | None = None, slopes: torch.Tensor | None = None,
-                    gate: torch.Tensor | None = None) -> "torch.Tensor | SplitAttention":
+                    gate: torch.Tensor | None = None, chunk_mask: int = 0) -> "torch.Tensor | SplitAttention":
     """Attention of a packed step over the cache; picks the kernel for the storage type and shape.
     float32 always takes the one-wave-per-row kernel, whose sums do not depend on the batch;
     bfloat16 takes the matrix-core kernels where they serve the shape. `leave_split`: a step of single
@@ -726,7 +733,12 @@ def paged_attention(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tenso
     back to `paged_attention_general`, which is 32-bit throughout. `sinks` / `slopes` (float32 [heads]): learned
     sinks (exp(sinks[h]) in the denominator) and a penalty of slopes[h] per position of distance on every score,
     by the general variants likewise. `gate` (float32 [tokens, heads * value_dim], rows may lie apart): the
-    output is multiplied element by element by sigmoid(gate) on its way out of whichever kernel writes it."""
+    output is multiplied element by element by sigmoid(gate) on its way out of whichever kernel writes it.
+    `chunk_mask` > 0 (instead of `window`): a position sees the keys of its own chunk of that many positions,
+    chunks counted from position 0 of the request; the kernels take it as a window below zero."""
+    _need(chunk_mask >= 0 and window >= 0 and not (chunk_mask and window), "a sliding window or chunks, both counted in positions")
+    if chunk_mask:
+        window = -chunk_mask
     general = softcap > 0 or sink or sinks is not None or slopes is not None or gate is not None
     extra = dict(softcap=softcap, sink=sink, sinks=sinks, slopes=slopes)
     tables = ctx.block_tables[space]
@@ -1724,12 +1736,12 @@ def _check_cache_pair(k_cache: torch.Tensor, v_cache: torch.Tensor, dtype: torch
 def qkv_finish(qkv: torch.Tensor, freqs: torch.Tensor | None, positions: torch.Tensor, slots: torch.Tensor | None,
                k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, num_heads: int, num_kv_heads: int,
                head_dim: int, value_dim: int, out_dtype: torch.dtype, *, interleaved: bool = True,
-               qk_norm_eps: float | None = None, v_norm_eps: float | None = None) -> torch.Tensor:
+               qk_norm_eps: float | None = None, v_norm_eps: float | None = None, amplitude: float = 1.0) -> torch.Tensor:
     """From a projected row q | k | v ([tokens, nh hd + nkv hd + nkv vd], float32 or `out_dtype`) to q
     [tokens, nh, hd] and the cache slots of k and v, in `out_dtype`. `freqs` (float64 [rot / 2]): q and
     k turn in their first rot dimensions by position * freqs[i], pair i being dimensions (2i, 2i+1) if
-    `interleaved`, else (i, i + rot/2). `qk_norm_eps` / `v_norm_eps`: each q and k head, and each value
-    head, is then divided by its root mean square (eps inside the root); None: not."""
+    `interleaved`, else (i, i + rot/2), cosine and sine times `amplitude`. `qk_norm_eps` / `v_norm_eps`: each q
+    and k head, and each value head, is then divided by its root mean square (eps inside the root); None: not."""
     _gpu(qkv, freqs, positions, slots, k_cache, v_cache)
     T = qkv.shape[0]
     row = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
@@ -1753,7 +1765,7 @@ def qkv_finish(qkv: torch.Tensor, freqs: torch.Tensor | None, positions: torch.T
         _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(qkv), _ptr(freqs), _ptr(positions), _ptr(slots), T, num_heads,
         num_kv_heads, head_dim, value_dim, rot, int(interleaved), int(qk_norm_eps is not None), float(qk_norm_eps or 0.0),
         int(v_norm_eps is not None), float(v_norm_eps or 0.0), page_size, *kst, *vst, _code(qkv.dtype), _code(out_dtype),
-        _stream()))
+        float(amplitude), _stream()))
     return q
 
 
@@ -1973,10 +1985,11 @@ MOE_MAX_TOP = 32
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | None, top: int, scale: float,
-              normalize: bool = True) -> tuple[torch.Tensor, torch.Tensor]:
+              normalize: bool = True, softmax_chosen: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
     """(experts int32 [tokens, top], weights float32 [tokens, top]): scores s = sigmoid(x · routerᵀ) in 32-bit;
     the `top` experts with the largest s + correction; weights s of the chosen, over their sum (+ 1e-20) if
-    `normalize`, times `scale`."""
+    `normalize`, times `scale`. `softmax_chosen`: the logits themselves are the scores, and the weights are the
+    softmax over the chosen experts' logits alone (times `scale`)."""
     _gpu(x, router, correction)
     _need(x.dim() == 2 and x.is_contiguous(), "the input must be contiguous [tokens, width]")
     E = router.shape[0]
@@ -1987,7 +2000,7 @@ def moe_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | 
     ids = torch.empty((x.shape[0], top), dtype=torch.int32, device=x.device)
     weights = torch.empty((x.shape[0], top), dtype=torch.float32, device=x.device)
     _run("moe_route", library().ts_moe_route(_ptr(ids), _ptr(weights), _ptr(x), _code(x.dtype), _ptr(router), _ptr(correction),
-                                             x.shape[0], x.shape[1], E, top, float(scale), int(normalize), _stream()))
+                                             x.shape[0], x.shape[1], E, top, float(scale), int(normalize), int(softmax_chosen), _stream()))
     return ids, weights
 
 
@@ -2024,12 +2037,15 @@ def moe_group(ids: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -
 
 
 def moe_gemm(x: torch.Tensor, weights: torch.Tensor, grouped: ExpertTiles, out_dtype: torch.dtype, *, per_token: bool,
-             glu: "tuple[float, float, float] | None" = None) -> torch.Tensor:
+             glu: "tuple[float, float, float] | None" = None, activation: str = "none") -> torch.Tensor:
     """out[pair] = x[row of the pair] · weights[expert of the pair]ᵀ for every pair of the step; `per_token`:
     x holds a row per token (a pair reads its token's), else a row per pair. weights [experts, n, k]; with
     `glu` = (limit, slope, up_shift) they hold gate rows then up rows (n = 2 ff) and the capped gated unit of
-    the two sums leaves: out [pairs, ff]."""
+    the two sums leaves: out [pairs, ff]. Without `glu`, `activation` "relu2" squares the sums' positive parts on
+    their way out."""
     _gpu(x, weights)
+    _need(activation in ("none", "relu2") and not (glu is not None and activation != "none"),
+          "ungated experts take no activation or the square of relu")
     P = grouped.sorted.shape[0]
     _need(x.dim() == 2 and x.is_contiguous() and x.shape[0] == (P // grouped.top if per_token else P), "the operand must be contiguous, a row per token or per pair")
     _need(weights.dim() == 3 and weights.is_contiguous() and weights.shape[0] == grouped.experts and weights.shape[2] == x.shape[1]
@@ -2045,7 +2061,7 @@ def moe_gemm(x: torch.Tensor, weights: torch.Tensor, grouped: ExpertTiles, out_d
     _need(grouped.tile_rows != MOE_LDS_TILE_ROWS or x.shape[1] % 64 == 0, "tiles of 128 rows: a reduction that is a multiple of 64")
     _run("moe_gemm", library().ts_moe_gemm(_ptr(out), _code(out_dtype), _ptr(x), _code(x.dtype), _ptr(weights), _ptr(grouped.sorted),
                                            _ptr(grouped.tiles), grouped.tiles.shape[0], grouped.tile_rows, grouped.top if per_token else 1, n, x.shape[1],
-                                           int(glu is not None), float(limit), float(slope), float(shift), _stream()))
+                                           int(glu is not None), float(limit), float(slope), float(shift), ACTIVATIONS[activation], _stream()))
     return out
 
 
@@ -2059,4 +2075,184 @@ def moe_combine(rows: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor 
           "the shared rows must be contiguous float32 [tokens, width]")
     out = torch.empty((T, rows.shape[1]), dtype=torch.float32, device=rows.device)
     _run("moe_combine", library().ts_moe_combine(_ptr(out), _ptr(rows), _ptr(weights), _ptr(shared), T, rows.shape[1], top, _stream()))
+    return out
+
+
+# ---- norms over stretches of rows, rotations of stretches of heads, per-head products ----
+
+def segment_rmsnorm(x: torch.Tensor, offset: int, size: int, weight: torch.Tensor | None, eps: float,
+                    out: torch.Tensor | None = None, out_dtype: torch.dtype = torch.float32) -> torch.Tensor:
+    """Columns [offset, offset + size) of every row of x (float32 [rows, width]) divided by their root mean square
+    (eps inside the root) times `weight` (float32 [size]; None: 1), 32-bit. `out` None: a new [rows, size] tensor
+    of `out_dtype`; `out` given (a view of x's own columns, say, to work in place): written there."""
+    _gpu(x, weight, out)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.stride(1) == 1, "rows of float32")
+    _need(0 <= offset and size > 0 and offset + size <= x.shape[1], "the stretch lies inside a row")
+    _need(weight is None or (weight.dtype == torch.float32 and weight.shape == (size,) and weight.is_contiguous()), "the weight must be float32 [size]")
+    if out is None:
+        out = torch.empty((x.shape[0], size), dtype=out_dtype, device=x.device)
+    _need(out.shape == (x.shape[0], size) and out.stride(1) == 1, "the output must be [rows, size]")
+    _run("segment_rmsnorm", library().ts_segment_rmsnorm(
+        _ptr(out), _code(out.dtype), out.stride(0) if x.shape[0] > 1 else size, x.data_ptr() + 4 * offset,
+        x.stride(0) if x.shape[0] > 1 else x.shape[1], size, _ptr(weight), float(eps), x.shape[0], _stream()))
+    return out
+
+
+def _check_step_vectors(T: int, **vectors: torch.Tensor | None) -> None:
+    for name, t in vectors.items():
+        _need(t is None or (t.dtype == torch.int32 and t.shape == (T,) and t.is_contiguous()), lambda: f"{name} must be int32 [tokens]")
+
+
+def _check_freqs(freqs: torch.Tensor | None, rot: int) -> None:
+    _need(rot % 2 == 0 and (rot == 0 or (freqs is not None and freqs.dtype == torch.float64 and freqs.shape == (rot // 2,)
+                                          and freqs.is_contiguous())), "frequencies must be float64 [rot / 2]")
+
+
+def _check_latent_cache(cache: torch.Tensor, row: int, dtype: torch.dtype) -> None:
+    _need(cache.dim() == 4 and cache.shape[2] == 1 and cache.shape[3] == row and cache.stride(3) == 1 and cache.dtype == dtype,
+          lambda: f"the latent cache view must be [pages, page_size, 1, {row}] of the step's storage type, got {tuple(cache.shape)}")
+
+
+LATENT_MAX_RANK = 512      # of a cached latent,
+LATENT_MAX_ROW = 640       # and of a cached row (latent and shared rotated key part)
+
+
+def latent_finish(down: torch.Tensor, q_off: int, q_rank: int, kv_off: int, rank: int, rot: int, q_weight: torch.Tensor | None,
+                  kv_weight: torch.Tensor, eps: float, freqs: torch.Tensor | None, amplitude: float, positions: torch.Tensor,
+                  slots: torch.Tensor | None, cache: torch.Tensor | None, out_dtype: torch.dtype) -> torch.Tensor | None:
+    """From the fused down-projection's rows (float32) to the query latent and the cache. Columns [q_off, + q_rank):
+    divided by their root mean square times `q_weight`, returned as [tokens, q_rank] of `out_dtype` (None if q_rank is
+    0). Columns [kv_off, + rank): likewise with `kv_weight`, the latent c; the next `rot` columns turn by the position
+    (pairs (2i, 2i+1), cosine and sine times `amplitude`); [c | turned] goes to the token's slot of `cache`."""
+    _gpu(down, q_weight, kv_weight, freqs, positions, slots, cache)
+    T = down.shape[0]
+    _need(down.dtype == torch.float32 and down.dim() == 2 and down.is_contiguous(), "the projected rows must be contiguous float32")
+    _need(q_rank == 0 or (q_weight is not None and q_weight.dtype == torch.float32 and q_weight.shape == (q_rank,) and q_weight.is_contiguous()),
+          "the query latent's weight must be float32 [q_rank]")
+    _need(kv_weight.dtype == torch.float32 and kv_weight.shape == (rank,) and kv_weight.is_contiguous(), "the latent's weight must be float32 [rank]")
+    _need(0 <= q_off and q_off + q_rank <= down.shape[1] and 0 <= kv_off and kv_off + rank + rot <= down.shape[1], "the stretches lie inside a row")
+    _check_freqs(freqs, rot)
+    _check_step_vectors(T, positions=positions, slots=slots)
+    page_size, kp, ks = 1, 0, 0
+    if cache is not None:
+        _need(slots is not None, "a cache write needs the slots")
+        _check_latent_cache(cache, rank + rot, out_dtype)
+        page_size, kp, ks = cache.shape[1], cache.stride(0), cache.stride(1)
+    cq = torch.empty((T, q_rank), dtype=out_dtype, device=down.device) if q_rank else None
+    _run("latent_finish", library().ts_latent_finish(
+        _ptr(cq), _ptr(cache), _code(out_dtype), _ptr(down), down.shape[1], q_off, q_rank, kv_off, rank, rot, _ptr(q_weight),
+        _ptr(kv_weight), float(eps), _ptr(freqs), float(amplitude), _ptr(positions), _ptr(slots), page_size, kp, ks, T, _stream()))
+    return cq
+
+
+def rotate_heads(dst: torch.Tensor, src: torch.Tensor, freqs: torch.Tensor, amplitude: float, positions: torch.Tensor,
+                 interleaved: bool = True) -> None:
+    """dst[t, h, :rot] = src[t, h, :rot] turned by positions[t] (rot = 2 len(freqs); pairs (2i, 2i+1) if `interleaved`,
+    else (i, i + rot/2); cosine and sine times `amplitude`). `src` float32 and `dst` are views [tokens, heads, >= rot]
+    whose last dimension is contiguous."""
+    _gpu(dst, src, freqs, positions)
+    T, H = src.shape[0], src.shape[1]
+    rot = 2 * freqs.shape[0]
+    _check_freqs(freqs, rot)
+    _check_step_vectors(T, positions=positions)
+    _need(src.dtype == torch.float32 and src.dim() == 3 and dst.dim() == 3 and dst.shape[:2] == src.shape[:2]
+          and src.shape[2] >= rot and dst.shape[2] >= rot and src.stride(2) == 1 and dst.stride(2) == 1, "views [tokens, heads, >= rot]")
+    _run("rotate_heads", library().ts_rotate_heads(
+        _ptr(dst), _code(dst.dtype), dst.stride(0), dst.stride(1), _ptr(src), src.stride(0), src.stride(1), H, rot, int(interleaved),
+        _ptr(freqs), float(amplitude), _ptr(positions), T, _stream()))
+
+
+def heads_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t, h, :] = x[t, h, :] · w[h] with w [heads, k, n] (any strides: a transposed view multiplies by the
+    transpose), 32-bit multiply-adds in ascending k. x [tokens, heads, k] and out [tokens, heads, n] are views whose
+    last dimension is contiguous. `gate` (float32 [tokens, heads * n], rows may lie apart): out is multiplied by
+    sigmoid(gate) on its way out."""
+    _gpu(x, w, out, gate)
+    T, H, K = x.shape
+    N = w.shape[2]
+    _need(w.dim() == 3 and w.shape[0] == H and w.shape[1] == K and out.shape == (T, H, N), "x [tokens, heads, k], w [heads, k, n], out [tokens, heads, n]")
+    _need(x.stride(2) == 1 and out.stride(2) == 1, "rows of x and out must be contiguous")
+    _run("heads_gemm", library().ts_heads_gemm(
+        _ptr(out), _code(out.dtype), out.stride(0), out.stride(1), _ptr(x), _code(x.dtype), x.stride(0), x.stride(1), _ptr(w),
+        _code(w.dtype), *w.stride(), T, H, N, K, _ptr(gate), _check_gate(gate, T, H * N), _stream()))
+    return out
+
+
+def paged_attention_latent(q: torch.Tensor, cache: torch.Tensor, rank: int, ctx, space: int, scale: float, window: int = 0,
+                           chunk_mask: int = 0, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """Multi-query attention of a packed step over cached rows [c | r] (c the first `rank` numbers, which are also
+    the values): q [tokens, heads, rank + rot] (float32, or the cache's type), out [tokens, heads, rank] = the softmax
+    weights' sum of c. Causal, with a sliding `window` or chunks (`chunk_mask`) as `paged_attention` has them."""
+    _gpu(q, cache)
+    _need(chunk_mask >= 0 and window >= 0 and not (chunk_mask and window), "a sliding window or chunks, both counted in positions")
+    T, H, row = q.shape
+    _need(q.is_contiguous() and 0 < rank <= min(row, LATENT_MAX_RANK) and row <= LATENT_MAX_ROW,
+          lambda: f"q must be contiguous [tokens, heads, rank + rot], rank up to {LATENT_MAX_RANK}, rows up to {LATENT_MAX_ROW}")
+    _check_latent_cache(cache, row, cache.dtype)
+    tables = ctx.block_tables[space]
+    table_page = getattr(ctx, "page_size", 0) or cache.shape[1]
+    _need(table_page % cache.shape[1] == 0, "block tables in whole pages of the cache")
+    _need(tables.dtype == torch.int32 and tables.dim() == 2 and tables.is_contiguous(), "block_tables must be contiguous int32 [requests, pages]")
+    _check_step_vectors(T, seq_of_token=ctx.seq_of_token, positions=ctx.positions)
+    out = torch.empty((T, H, rank), dtype=out_dtype or cache.dtype, device=q.device)
+    _run("paged_attention_latent", library().ts_paged_attention_latent(
+        _ptr(out), _code(out.dtype), _ptr(q), _code(q.dtype), _ptr(cache), _code(cache.dtype), _ptr(tables), _ptr(ctx.seq_of_token),
+        _ptr(ctx.positions), T, H, rank, row - rank, cache.shape[1], cache.stride(0), cache.stride(1), tables.shape[1], float(scale),
+        -chunk_mask if chunk_mask else int(window), _page_run(table_page // cache.shape[1]), _stream()))
+    return out
+
+
+# ---- mLSTM ----
+
+MLSTM_MAX_DIM = 1024
+MLSTM_ROWS_PER_THREAD = 32     # rows of a head's state that a thread keeps of its column, where the column count allows
+
+
+def mlstm_columns(dim: int, vdim: int) -> int:
+    """Value columns per workgroup of the scan: as many as leave a thread at most `MLSTM_ROWS_PER_THREAD` rows of the
+    state (256 threads, a column's rows spread over 256 // columns of them)."""
+    cols = min(vdim, 256)
+    while cols > 16 and -(-dim // (256 // cols)) > MLSTM_ROWS_PER_THREAD:
+        cols = -(-cols // 2)
+    return cols
+
+
+def mlstm_state_size(heads: int, dim: int, vdim: int) -> int:
+    """Floats of a request's state: per head S [dim, vdim], n [dim] and m."""
+    return heads * (dim * vdim + dim + 1)
+
+
+def mlstm_scan(proj: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor,
+               state_slots: torch.Tensor, heads: int, dim: int, vdim: int, cap: float) -> torch.Tensor:
+    """The recurrence over a packed step. proj float32 [tokens, >= 2 heads dim + heads vdim + 2 heads]: per token
+    q | k | v | the input gates' sums | the forget gates' sums (then whatever else the fused projection makes); state
+    float32 [slots, heads (dim vdim + dim + 1)], read at each request's slot and written back. Returns o float32
+    [tokens, heads vdim], before the heads' norm."""
+    _gpu(proj, i_bias, f_bias, state, cu_seqlens, state_slots)
+    T = proj.shape[0]
+    need = 2 * heads * dim + heads * vdim + 2 * heads
+    _need(proj.dtype == torch.float32 and proj.dim() == 2 and proj.is_contiguous() and proj.shape[1] >= need, "the projected rows must be contiguous float32")
+    for b in (i_bias, f_bias):
+        _need(b.dtype == torch.float32 and b.shape == (heads,) and b.is_contiguous(), "a gate's bias must be float32 [heads]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] == mlstm_state_size(heads, dim, vdim) and state.is_contiguous(),
+          "the state must be contiguous float32 [slots, heads (dim vdim + dim + 1)]")
+    S = state_slots.shape[0]
+    _need(cu_seqlens.dtype == torch.int32 and cu_seqlens.shape == (S + 1,) and state_slots.dtype == torch.int32, "cu_seqlens int32 [requests + 1], slots int32 [requests]")
+    _need(0 < dim <= MLSTM_MAX_DIM and cap > 0, lambda: f"heads of up to {MLSTM_MAX_DIM} dimensions, a positive cap")
+    out = torch.empty((T, heads * vdim), dtype=torch.float32, device=proj.device)
+    _run("mlstm_scan", library().ts_mlstm_scan(_ptr(out), _ptr(proj), proj.shape[1], _ptr(i_bias), _ptr(f_bias), _ptr(state), _ptr(cu_seqlens),
+                                               _ptr(state_slots), S, heads, dim, vdim, mlstm_columns(dim, vdim), float(cap), float(dim) ** -0.5, _stream()))
+    return out
+
+
+def mlstm_finish(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, heads: int, vdim: int, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """Each head's row of o (float32 [tokens, heads vdim]) divided by its root mean square, times `weight` (float32
+    [heads vdim]), times sigmoid(gate) (float32 [tokens, heads vdim], rows may lie apart), as `out_dtype`."""
+    _gpu(o, weight, gate)
+    T = o.shape[0]
+    _need(o.dtype == torch.float32 and o.shape == (T, heads * vdim) and o.is_contiguous(), "o must be contiguous float32 [tokens, heads vdim]")
+    _need(weight.dtype == torch.float32 and weight.shape == (heads * vdim,) and weight.is_contiguous(), "the weight must be float32 [heads vdim]")
+    out = torch.empty((T, heads * vdim), dtype=out_dtype, device=o.device)
+    _run("mlstm_finish", library().ts_mlstm_finish(_ptr(out), _code(out_dtype), _ptr(o), _ptr(weight), _ptr(gate), _check_gate(gate, T, heads * vdim),
+                                                   T, heads, vdim, float(eps), _stream()))
     return out

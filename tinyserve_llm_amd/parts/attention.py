@@ -139,7 +139,17 @@ class GeneralAttention(Mixer):
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int | None = None,
                  position: str | None = None, scale: float | None = None, softcap: float = 0.0, sink: bool = False,
-                 qk_norm_eps: float | None = None, v_norm_eps: float | None = None, window: int = 0) -> None:
+                 qk_norm_eps: float | None = None, v_norm_eps: float | None = None, window: int = 0, chunk: int = 0,
+                 learned_sink: bool = False, projection_norm_eps: float | None = None) -> None:
+        """Further options. `chunk` (instead of `window`): a position sees the keys of its own chunk of that many
+        positions, chunks counted from position 0. `learned_sink`: exp(sink[h]), a learned number per head, in the
+        softmax's denominator (instead of `sink`'s 1). `projection_norm_eps`: the whole q projection of a token (all
+        heads at once), and likewise the whole k projection, is divided by its root mean square and multiplied by a
+        weight of that size (`q_norm`, `k_norm`, 32-bit) before the heads turn."""
+        if chunk < 0 or window < 0 or (chunk and window):
+            raise ValueError("a sliding window or chunks (both >= 0), not both")
+        if sink and learned_sink:
+            raise ValueError("a sink of score 0 or a learned one, not both")
         if num_heads % num_kv_heads:
             raise ValueError(f"{num_heads} heads do not divide into {num_kv_heads} key/value heads")
         value_dim = head_dim if value_dim is None else value_dim
@@ -151,8 +161,12 @@ class GeneralAttention(Mixer):
         self.head_dim, self.value_dim, self.position = head_dim, value_dim, position
         self.scale = scale if scale is not None else head_dim ** -0.5
         self.softcap, self.sink, self.qk_norm_eps, self.v_norm_eps, self.window = softcap, sink, qk_norm_eps, v_norm_eps, window
+        self.chunk, self.learned_sink, self.projection_norm_eps = chunk, learned_sink, projection_norm_eps
         self.qkv: torch.Tensor | None = None
         self.o: torch.Tensor | None = None
+        self.q_norm: torch.Tensor | None = None
+        self.k_norm: torch.Tensor | None = None
+        self.sinks: torch.Tensor | None = None
         self.qkv_packed: hip.StreamingCopies | None = None
         self.o_packed: hip.StreamingCopies | None = None
 
@@ -169,11 +183,18 @@ class GeneralAttention(Mixer):
         return self.num_kv_heads * self.value_dim
 
     def param_specs(self) -> dict[str, ParamSpec]:
-        return {"qkv": ParamSpec((self.q_size + self.k_size + self.v_size, self.hidden_size)),
-                "o": ParamSpec((self.hidden_size, self.num_heads * self.value_dim))}
+        specs = {"qkv": ParamSpec((self.q_size + self.k_size + self.v_size, self.hidden_size)),
+                 "o": ParamSpec((self.hidden_size, self.num_heads * self.value_dim))}
+        if self.projection_norm_eps is not None:
+            specs["q_norm"] = ParamSpec((self.q_size,), "float32", init=(1.0, 0.1))
+            specs["k_norm"] = ParamSpec((self.k_size,), "float32", init=(1.0, 0.1))
+        if self.learned_sink:
+            specs["sinks"] = ParamSpec((self.num_heads,), "float32", init=(0.0, 1.0))
+        return specs
 
     def kv_spec(self) -> KVSpec:
-        return KVSpec(self.num_kv_heads, self.head_dim, self.window,
+        # (a chunk's keys lie within the last `chunk` positions: the cache may give back what lies before them)
+        return KVSpec(self.num_kv_heads, self.head_dim, self.window or self.chunk,
                       None if self.value_dim == self.head_dim else self.value_dim)
 
     def keep_streaming_copies(self) -> int:
@@ -185,12 +206,16 @@ class GeneralAttention(Mixer):
         slots = ctx.slot_mapping[mem.space] if mem.store else None
         k_store, v_store = (mem.k_cache, mem.v_cache) if mem.store else (None, None)
         qkv = linear(x, self.qkv, out_dtype=torch.float32, packed=self.qkv_packed)
+        if self.projection_norm_eps is not None:         # in place, each over its whole stretch of the row
+            hip.segment_rmsnorm(qkv, 0, self.q_size, self.q_norm, self.projection_norm_eps, out=qkv[:, :self.q_size])
+            hip.segment_rmsnorm(qkv, self.q_size, self.k_size, self.k_norm, self.projection_norm_eps,
+                                out=qkv[:, self.q_size:self.q_size + self.k_size])
         q = hip.qkv_finish(qkv, enc.frequencies() if enc is not None else None, ctx.positions, slots, k_store, v_store,
                            self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, x.dtype,
                            interleaved=getattr(enc, "interleaved", True), qk_norm_eps=self.qk_norm_eps,
-                           v_norm_eps=self.v_norm_eps)
+                           v_norm_eps=self.v_norm_eps, amplitude=getattr(enc, "amplitude", 1.0))
         o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window, softcap=self.softcap,
-                                sink=self.sink)
+                                sink=self.sink, sinks=self.sinks, chunk_mask=self.chunk)
         return linear(o.view(ctx.num_tokens, self.num_heads * self.value_dim), self.o, out_dtype=torch.float32,
                       packed=self.o_packed)
 

@@ -154,3 +154,24 @@ def sandwich_block(layer: Layer, hidden, residual, ctx: StepContext, mem: LayerM
         return stream, None
     x, h = stream.take(norms["norm2"], out_dtype=norms["norm2"].weight.dtype)
     return ResidualStream(x, layer.feed_forward.forward(h, ctx), post=norms["norm2b"]), None
+
+
+@register("block", "pre_norm_stream")
+@uses_norms("norm1")
+@keeps_stream
+def pre_norm_stream_block(layer: Layer, hidden, residual, ctx: StepContext, mem: LayerMemory):
+    """x <- x + mixer(norm1(x)), then x <- x + feed_forward(norm2(x)) on a 32-bit residual stream ("norm2" only where
+    the layer has a feed-forward). Each sum is left pending in the stream, so that the norm that reads the stream
+    next (this layer's second, the next layer's first, or the model's last) is made by the kernel that adds."""
+    from tinyserve_llm_amd.parts.stream import ResidualStream
+    if not isinstance(hidden, ResidualStream) or residual is not None:
+        raise TypeError("this arrangement runs on a 32-bit residual stream (ModelSpec.residual_dtype = 'float32')")
+    norms = layer.norms
+    x, h = hidden.take(norms["norm1"])
+    stream = ResidualStream(x, layer.mixer.forward(h, ctx, mem))
+    if "norm2" not in norms:
+        if layer.feed_forward.forward(None, ctx) is not None:
+            raise KeyError("a layer with a feed-forward names the norm 'norm2'")
+        return stream, None
+    x, h = stream.take(norms["norm2"])
+    return ResidualStream(x, layer.feed_forward.forward(h, ctx)), None

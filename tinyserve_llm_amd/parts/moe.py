@@ -70,3 +70,44 @@ class RoutedExperts(FeedForward):
         rows = hip.moe_gemm(unit, self.down, grouped, torch.float32, per_token=False)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
         return hip.moe_combine(rows, weights, shared)
+
+
+@register("feed_forward", "routed_dense_experts")
+class RoutedDenseExperts(FeedForward):
+    """Experts without a gate and without biases: W_down act(W_up h), `activation` "relu2" (the square of relu) or
+    "none". Router logits z = W_r h in 32-bit; the `top` experts with the largest logits are chosen and their weights
+    are the softmax over the chosen logits alone (`scoring` "softmax_chosen"), or sigmoid scores normalised over the
+    chosen (`scoring` "sigmoid"), times `router_scale`. The experts' matrices are stacked: up [experts, ff, hidden],
+    down [experts, hidden, ff]; the activation rides on the up product's way out, the down product and the weighted
+    sum are 32-bit."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, num_experts: int, top: int, intermediate_size: int, activation: str = "relu2",
+                 scoring: str = "softmax_chosen", router_scale: float = 1.0) -> None:
+        if not 1 <= top <= min(num_experts, hip.MOE_MAX_TOP) or num_experts > hip.MOE_MAX_EXPERTS:
+            raise ValueError(f"top {top} of {num_experts} experts: 1 <= top <= min(experts, {hip.MOE_MAX_TOP}), "
+                             f"experts <= {hip.MOE_MAX_EXPERTS}")
+        if activation not in ("relu2", "none") or scoring not in ("softmax_chosen", "sigmoid"):
+            raise ValueError("activation 'relu2' or 'none'; scoring 'softmax_chosen' or 'sigmoid'")
+        self.hidden_size, self.num_experts, self.top, self.intermediate_size = hidden_size, num_experts, top, intermediate_size
+        self.activation, self.scoring, self.router_scale = activation, scoring, router_scale
+        self.router: torch.Tensor | None = None
+        self.up: torch.Tensor | None = None
+        self.down: torch.Tensor | None = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        E, F, H = self.num_experts, self.intermediate_size, self.hidden_size
+        return {"router": ParamSpec((E, H), "float32", init=(0.0, 0.2)), "up": ParamSpec((E, F, H)), "down": ParamSpec((E, H, F))}
+
+    def widest_activation(self) -> int:
+        return max(2 * self.top * self.hidden_size, self.top * self.intermediate_size)
+
+    def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        experts, weights = hip.moe_route(x, self.router, None, self.top, self.router_scale, True,
+                                         softmax_chosen=self.scoring == "softmax_chosen")
+        tile_rows = hip.moe_tile_rows(experts.numel(), self.num_experts, x.dtype, (self.hidden_size, self.intermediate_size))
+        grouped = hip.moe_group(experts, self.num_experts, tile_rows)
+        act = hip.moe_gemm(x, self.up, grouped, x.dtype, per_token=True, activation=self.activation)
+        rows = hip.moe_gemm(act, self.down, grouped, torch.float32, per_token=False)
+        return hip.moe_combine(rows, weights, None)

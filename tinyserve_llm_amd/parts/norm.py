@@ -19,20 +19,30 @@ from tinyserve_llm_amd.parts.stream import ResidualStream
 class RMSNorm(Norm):
     graph_safe = True
 
-    def __init__(self, hidden_size: int, eps: float) -> None:
+    def __init__(self, hidden_size: int, eps: float, one_plus: bool = False) -> None:
+        """`one_plus`: the weight is stored around zero and the rows are multiplied by 1 + weight (the sum taken
+        in 32-bit, once, when the weights arrive); such a norm works on a 32-bit residual stream."""
         self.hidden_size = hidden_size
         self.eps = eps
+        self.one_plus = one_plus
         self.weight: torch.Tensor | None = None
+        self.applied: torch.Tensor | None = None      # what the rows are multiplied by: the weight, or 1 + weight in 32-bit
 
     def param_specs(self) -> dict[str, ParamSpec]:
-        return {"weight": ParamSpec((self.hidden_size,), init=(1.0, 0.1))}
+        return {"weight": ParamSpec((self.hidden_size,), init=(0.0, 0.1) if self.one_plus else (1.0, 0.1))}
+
+    def bind(self, params) -> None:
+        super().bind(params)
+        self.applied = (1.0 + self.weight.float()).contiguous() if self.one_plus else self.weight
 
     def __call__(self, x, residual=None, rows=None):
         if isinstance(x, ResidualStream):
             # a 32-bit stream: its pending sum, then the norm, rounded to the weights' storage type on the way out
             if residual is not None:
                 raise ValueError("a residual stream carries its own sum")
-            return x.norm_rows(rows, self.weight, self.eps, self.weight.dtype), (None if rows is not None else x.x)
+            return x.norm_rows(rows, self.applied, self.eps, self.weight.dtype), (None if rows is not None else x.x)
+        if self.one_plus:
+            raise TypeError("a norm with 1 + weight works on a 32-bit residual stream (ModelSpec.residual_dtype = 'float32')")
         return hip.rmsnorm(x, self.weight, self.eps, residual, rows)
 
     def defer(self, x, residual=None) -> DeferredNorm:

@@ -71,15 +71,35 @@ class RotaryFrequencies(PositionEncoding):
 
     graph_safe = True
 
-    def __init__(self, rotary_dim: int, theta: float, interleaved: bool = True) -> None:
+    def __init__(self, rotary_dim: int, theta: float, interleaved: bool = True, ramp: dict | None = None) -> None:
+        """`ramp` (factor s, original length L, fast, slow): frequencies are slowed down by s along a ramp over
+        the pairs: with d(t) = rotary_dim ln(L / (2 pi t)) / (2 ln theta), lo = max(floor d(fast), 0),
+        hi = min(ceil d(slow), rotary_dim - 1) and r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), pair i
+        turns with f_i / s * r_i + f_i (1 - r_i), and cosine and sine are multiplied by `amplitude` =
+        0.1 ln s + 1 (the mixers' kernels take it beside the frequencies)."""
         if rotary_dim % 2 or rotary_dim < 0:
             raise ValueError(f"rotary_dim {rotary_dim}: an even number of dimensions turns")
         self.rotary_dim, self.theta, self.interleaved = rotary_dim, float(theta), interleaved
+        self.ramp = dict(ramp) if ramp else None
+        if self.ramp is not None and not (self.ramp["factor"] > 0 and self.ramp["original"] > 0 and self.ramp["fast"] > 0
+                                          and self.ramp["slow"] > 0 and self.theta > 1):
+            raise ValueError("a frequency ramp needs positive factor, original, fast and slow, and a base above 1")
+        self.amplitude = 0.1 * math.log(self.ramp["factor"]) + 1.0 if self.ramp is not None else 1.0
         self.freqs: torch.Tensor | None = None
 
     def host_frequencies(self) -> torch.Tensor:
         i = torch.arange(self.rotary_dim // 2, dtype=torch.float64)
-        return torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / max(1, self.rotary_dim))
+        f = torch.pow(torch.tensor(self.theta, dtype=torch.float64), -2.0 * i / max(1, self.rotary_dim))
+        if self.ramp is None:
+            return f
+        r = self.ramp
+
+        def crossing(turns: float) -> float:
+            return self.rotary_dim * math.log(r["original"] / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+        lo, hi = max(math.floor(crossing(r["fast"])), 0), min(math.ceil(crossing(r["slow"])), self.rotary_dim - 1)
+        ramp = torch.clamp((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+        return f / r["factor"] * ramp + f * (1.0 - ramp)
 
     def prepare(self, device: torch.device) -> None:
         self.freqs = self.host_frequencies().to(device) if self.rotary_dim else None
