@@ -99,3 +99,43 @@ def fanotar_configs():
     S = FanotarConfig(vocab=300, width=512, norm_eps=1e-6, embedding_scale=12.0, layers=(
         L(d0, E(experts=8, top=2, scale=1.5, expert=U(128, 2.0), shared=U(256, 1.0))), L(d1, U(640, 2.0))))
     return {"P": (P, 3), "Q": (Q, 4), "R": (R, 5), "S": (S, 6)}
+
+
+def bafarax_configs():
+    """Small Bafarax configurations that differ from each other in every size and option: the order of the three
+    mixers, key/value grouping, key and value head sizes (equal or not), how much of a head turns (all, part, none),
+    frequency ramps or none, chunks and windows (one position, shorter and longer than a page, none), latents larger
+    and smaller than the heads they feed, an mLSTM whose values span several workgroups, layers that run with an
+    earlier layer's weights, dense, routed (one expert per token up to all of them) and absent feed-forwards, an
+    embedding scale of 1, and widths that are multiples of nothing."""
+    from tinyserve_llm_amd.config.bafarax import BafaraxAttention as A, BafaraxConfig, BafaraxDense as D, BafaraxExperts as E, \
+        BafaraxLatentAttention as LA, BafaraxLayer as L, BafaraxMLSTM as M, FrequencyRamp as Ramp, Rotation as Rot
+    p_att = A(heads=4, kv_heads=2, dim=32, vdim=48, scale=0.3, rot=Rot(16, 10000.0), chunk=24)
+    p_lat = LA(heads=3, dim=24, rot_dim=8, vdim=20, kv_rank=40, q_rank=36, scale=0.2,
+               rot=Rot(8, 5000.0, Ramp(factor=3.0, original=64.0, fast=16.0, slow=2.0)), window=50)
+    P = BafaraxConfig(vocab=200, width=80, norm_eps=1e-6, embedding_scale=7.0, layers=(
+        L("mlstm", M(heads=3, dim=20, vdim=28, gate_cap=8.0), D(96)), L("attention", p_att, E(experts=6, top=3, ff=40)),
+        L("latent_attention", p_lat, None), L("attention", p_att, E(experts=6, top=3, ff=40), weights_of=1)))
+    q_att = A(heads=2, kv_heads=2, dim=16, vdim=16, scale=0.25, rot=Rot(16, 700.0), chunk=1)
+    q_lat = LA(heads=2, dim=16, rot_dim=16, vdim=16, kv_rank=16, q_rank=16, scale=0.4, rot=Rot(16, 300.0), window=70)
+    q_mem = M(heads=1, dim=16, vdim=16, gate_cap=15.0)
+    q_full = A(heads=4, kv_heads=1, dim=8, vdim=24, scale=0.35, rot=Rot(0, 1.0), chunk=0)
+    Q = BafaraxConfig(vocab=131, width=48, norm_eps=1e-4, embedding_scale=1.0, layers=(
+        L("attention", q_att, E(experts=4, top=1, ff=20)), L("latent_attention", q_lat, D(64)), L("mlstm", q_mem, None),
+        L("mlstm", q_mem, None, weights_of=2), L("latent_attention", q_lat, D(64), weights_of=1),
+        L("attention", q_full, E(experts=3, top=3, ff=12))))
+    # sizes that are multiples of nothing in particular: no kernel's fast path takes them
+    r_lat = LA(heads=3, dim=20, rot_dim=6, vdim=12, kv_rank=34, q_rank=22, scale=0.3,
+               rot=Rot(6, 2000.0, Ramp(factor=8.0, original=32.0, fast=4.0, slow=1.0)), window=7)
+    R = BafaraxConfig(vocab=77, width=99, norm_eps=1e-5, embedding_scale=3.5, layers=(
+        L("latent_attention", r_lat, E(experts=5, top=2, ff=17)),
+        L("attention", A(heads=3, kv_heads=1, dim=20, vdim=12, scale=0.3, rot=Rot(10, 50000.0), chunk=50), D(52)),
+        L("mlstm", M(heads=2, dim=18, vdim=270, gate_cap=5.0), D(40))))
+    # a width that the weight-streaming kernels take, heads of a matrix-core size, experts in tiles of several rows
+    s_att = A(heads=8, kv_heads=2, dim=64, vdim=64, scale=0.11, rot=Rot(32, 250000.0), chunk=33)
+    S = BafaraxConfig(vocab=300, width=512, norm_eps=1e-6, embedding_scale=12.0, layers=(
+        L("attention", s_att, E(experts=8, top=2, ff=128)),
+        L("latent_attention", LA(heads=8, dim=64, rot_dim=32, vdim=64, kv_rank=256, q_rank=192, scale=0.1, rot=Rot(32, 10000.0),
+                                 window=130), D(640)),
+        L("mlstm", M(heads=4, dim=64, vdim=128, gate_cap=12.0), D(640)), L("attention", s_att, E(experts=8, top=2, ff=128), weights_of=0)))
+    return {"P": (P, 3), "Q": (Q, 4), "R": (R, 5), "S": (S, 6)}

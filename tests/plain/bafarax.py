@@ -200,10 +200,6 @@ def expert_mixture(h: torch.Tensor, W: dict, mlp: dict) -> torch.Tensor:
     return out
 
 
-def gelu_tanh(z: torch.Tensor) -> torch.Tensor:
-    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z ** 3)))
-
-
 class PlainBafarax:
     """The whole decoder over one request, fed in any portions; keeps that request's caches and states."""
 
@@ -253,3 +249,26 @@ class PlainBafarax:
                 x = x + (gated_unit(h, F) if mlp["kind"] == "dense" else expert_mixture(h, F, mlp))
             self.after_layers.append(x.clone())
         return layer_norm(x, self.w["final.norm"], eps) @ self.w["head"].T
+
+    def reset(self) -> None:
+        """Forgets the request: the next tokens are a new request's first."""
+        self.memory = [dict() for _ in self.c["layers"]]
+        self.fed = 0
+
+    def logits(self, tokens: list[int]) -> torch.Tensor:
+        """[len(tokens), vocab] for a request of its own, fed whole."""
+        self.reset()
+        return self.forward(tokens)
+
+    def streams(self, tokens: list[int]) -> list[torch.Tensor]:
+        """The residual stream after every layer, for a request of its own, fed whole."""
+        self.logits(tokens)
+        return self.after_layers
+
+    def greedy(self, tokens: list[int], n: int) -> list[int]:
+        self.reset()
+        row, out = self.forward(tokens)[-1], []
+        for _ in range(n):
+            out.append(int(row.argmax()))
+            row = self.forward(out[-1:])[-1]
+        return out
