@@ -30,6 +30,14 @@ reading its neighbour's cache, capped gated feed-forward, dense and as a mixture
 the Rugezen decoder, the closest of the engine's models, at equal layer sizes and equal active parameters
 per token, in the same way: whole-engine throughput and the like kernels side by side. One JSON line.
 
+    python bench.py --bafarax [--shape 1b|3b] [--layers L] [--kernels-only]
+
+measures the Bafarax decoder (pre-norm layers on a 32-bit stream whose mixers are, in turn, attention inside chunks
+with a norm over the whole projections and learned sinks, attention through a low-rank latent with a window and an
+output gate, and an mLSTM's matrix memory; dense and ungated routed feed-forwards) beside the Fanotar decoder, the
+closest of the engine's models, at equal layer sizes and equal active parameters per token, in the same way. One JSON
+line.
+
     python bench.py --scenario requests-3b | chunked-8b [--layers L]
 
 runs a whole workload through `LLM.generate` instead and prints one JSON line of its own: many
@@ -348,48 +356,30 @@ def designs(args) -> int:
     return 0
 
 
-def fanotar(args) -> int:
-    """The Fanotar decoder beside the Rugezen decoder at the layer sizes of `--shape`: whole-engine
-    throughput, and the like kernels of the two side by side. One JSON line."""
-    import torch
+class DesignBench:
+    """What the comparisons of two designs share: whole-engine throughput of a configuration with random weights,
+    a kernel's time from replays of a graph with cold caches, and a packed step's context over pages of its own."""
 
-    from tinyserve_llm_amd.config.fanotar import FanotarAttention, FanotarConfig, FanotarExperts, FanotarGatedUnit, FanotarLayer
-    from tinyserve_llm_amd.config.rugezen import RugezenAttention, RugezenConfig, RugezenLayer
-    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
-    from tinyserve_llm_amd.engine.loading import random_model
-    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
-    from tinyserve_llm_amd.engine.sequence import SamplingParams
-    from tinyserve_llm_amd.ops import hip
-    from tinyserve_llm_amd.parts.base import StepContext
-    from tinyserve_llm_amd.parts.linear import linear
+    def __init__(self, vocab: int, prompt_len: int) -> None:
+        import torch
+        self.vocab, self.prompt_len = vocab, prompt_len
+        self.max_model_len = max(MAX_MODEL_LEN, prompt_len + 1024)
+        self.rng = random.Random(0)
+        self.begin, self.end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        self.sweep = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
+        self.overhead: list[float] = []
 
-    sizes = SHAPES[args.shape]
-    sh = sizes["shape"]
-    layers = args.layers or sizes["layers_full"]
-    hidden, nh, nkv, hd, inter, vocab = (sh["hidden_size"], sh["num_attention_heads"], sh["num_key_value_heads"], sh["head_dim"],
-                                         sh["intermediate_size"], sh["vocab_size"])
-    window, taps, experts, top = 1024, 4, 16, 4
-    eff, sff = inter // 8, inter // 2                 # four experts of an eighth and a shared half: one dense width per token
-    ratt = RugezenAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, rot_dims=hd // 2, rot_base=1.0e6, scale=hd ** -0.5, softcap=30.0)
-    rug = RugezenConfig(vocab=vocab, width=hidden, norm_eps=1e-6, residual_mult=0.6,
-                        layers=tuple(RugezenLayer("attention", ratt, 3 * inter // 2) for _ in range(layers)))
-
-    def fan_layer(i):
-        att = FanotarAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, conv=taps, window=window, scale=hd ** -0.5, q_temp_coef=0.1,
-                               q_temp_every=1024, kv_from=i - 1 if i % 4 == 3 else None)
-        dense = FanotarGatedUnit(inter, 7.0)
-        moe = FanotarExperts(experts=experts, top=top, scale=2.5, expert=FanotarGatedUnit(eff, 7.0), shared=FanotarGatedUnit(sff, 7.0))
-        return FanotarLayer(att, moe if i % 2 else dense)
-    fan = FanotarConfig(vocab=vocab, width=hidden, norm_eps=1e-6, embedding_scale=float(hidden) ** 0.5,
-                        layers=tuple(fan_layer(i) for i in range(layers)))
-    prompt_len = args.context
-    max_model_len = max(MAX_MODEL_LEN, prompt_len + 1024)
-    rng = random.Random(0)
-    begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-
-    def whole_engine(config) -> dict:
-        model = random_model(config, 0, torch.bfloat16, "cuda:0")
+    def whole_engine(self, config) -> dict:
         import math
+
+        import torch
+
+        from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+        from tinyserve_llm_amd.engine.loading import random_model
+        from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+        from tinyserve_llm_amd.engine.sequence import SamplingParams
+        vocab, prompt_len, max_model_len, rng = self.vocab, self.prompt_len, self.max_model_len, self.rng
+        model = random_model(config, 0, torch.bfloat16, "cuda:0")
         out = {"parameters": sum(math.prod(ps.shape) for name, ps in model.param_specs().items() if name.startswith("layers."))}
 
         def engine(batch):
@@ -430,10 +420,8 @@ def fanotar(args) -> int:
         torch.cuda.empty_cache()
         return out
 
-    sweep = torch.zeros(128 << 20, dtype=torch.int32, device="cuda")
-    overhead = []
-
-    def replayed(fn, reps: int) -> float:
+    def replayed(self, fn, reps: int) -> float:
+        import torch
         fn()
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
@@ -441,27 +429,31 @@ def fanotar(args) -> int:
             kept = fn()
         best = float("inf")
         for _ in range(reps):
-            sweep.sum()
-            begin.record()
+            self.sweep.sum()
+            self.begin.record()
             graph.replay()
-            end.record()
-            end.synchronize()
-            best = min(best, 1e3 * begin.elapsed_time(end))
+            self.end.record()
+            self.end.synchronize()
+            best = min(best, 1e3 * self.begin.elapsed_time(self.end))
         del kept, graph
         return best
 
-    def timed(fn, reps: int = 5) -> float:
+    def timed(self, fn, reps: int = 5) -> float:
         """Microseconds of the best replay of `fn` recorded into a graph, each after a sweep of the caches,
         less what the replay of a graph of one tiny kernel takes."""
-        if not overhead:
+        import torch
+        if not self.overhead:
             tiny = torch.zeros(64, dtype=torch.int32, device="cuda")
-            overhead.append(replayed(lambda: tiny.add_(1), reps))
-        return max(replayed(fn, reps) - overhead[0], 1e-3)
+            self.overhead.append(self.replayed(lambda: tiny.add_(1), reps))
+        return max(self.replayed(fn, reps) - self.overhead[0], 1e-3)
 
-    dev = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
-    bf = torch.bfloat16
+    def context(self, starts, counts, pool_page):
+        """(a packed step in which request i feeds `counts[i]` tokens from position `starts[i]` over pages of its own,
+        its cache slots, the pool pages of `pool_page` tokens that takes)."""
+        import torch
 
-    def context(starts, counts, pool_page):
+        from tinyserve_llm_amd.parts.base import StepContext
+        dev = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
         positions, seq_of, cu, tables = [], [], [0], []
         per = -(-max(a + b for a, b in zip(starts, counts)) // PAGE)
         for i, (s0, n) in enumerate(zip(starts, counts)):
@@ -476,6 +468,47 @@ def fanotar(args) -> int:
                           slot_mapping=[slots], block_tables=[dev(tables)], host_cu_seqlens=cu, host_starts=list(starts),
                           host_context_lens=ends, host_state_slots=list(range(len(starts))), page_size=PAGE)
         return ctx, slots, len(starts) * per * (PAGE // pool_page)
+
+
+def fanotar(args) -> int:
+    """The Fanotar decoder beside the Rugezen decoder at the layer sizes of `--shape`: whole-engine
+    throughput, and the like kernels of the two side by side. One JSON line."""
+    import torch
+
+    from tinyserve_llm_amd.config.fanotar import FanotarAttention, FanotarConfig, FanotarExperts, FanotarGatedUnit, FanotarLayer
+    from tinyserve_llm_amd.config.rugezen import RugezenAttention, RugezenConfig, RugezenLayer
+    from tinyserve_llm_amd.engine.llm import LLM, CacheConfig
+    from tinyserve_llm_amd.engine.loading import random_model
+    from tinyserve_llm_amd.engine.scheduler import SchedulerConfig
+    from tinyserve_llm_amd.engine.sequence import SamplingParams
+    from tinyserve_llm_amd.ops import hip
+    from tinyserve_llm_amd.parts.base import StepContext
+    from tinyserve_llm_amd.parts.linear import linear
+
+    sizes = SHAPES[args.shape]
+    sh = sizes["shape"]
+    layers = args.layers or sizes["layers_full"]
+    hidden, nh, nkv, hd, inter, vocab = (sh["hidden_size"], sh["num_attention_heads"], sh["num_key_value_heads"], sh["head_dim"],
+                                         sh["intermediate_size"], sh["vocab_size"])
+    window, taps, experts, top = 1024, 4, 16, 4
+    eff, sff = inter // 8, inter // 2                 # four experts of an eighth and a shared half: one dense width per token
+    ratt = RugezenAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, rot_dims=hd // 2, rot_base=1.0e6, scale=hd ** -0.5, softcap=30.0)
+    rug = RugezenConfig(vocab=vocab, width=hidden, norm_eps=1e-6, residual_mult=0.6,
+                        layers=tuple(RugezenLayer("attention", ratt, 3 * inter // 2) for _ in range(layers)))
+
+    def fan_layer(i):
+        att = FanotarAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, conv=taps, window=window, scale=hd ** -0.5, q_temp_coef=0.1,
+                               q_temp_every=1024, kv_from=i - 1 if i % 4 == 3 else None)
+        dense = FanotarGatedUnit(inter, 7.0)
+        moe = FanotarExperts(experts=experts, top=top, scale=2.5, expert=FanotarGatedUnit(eff, 7.0), shared=FanotarGatedUnit(sff, 7.0))
+        return FanotarLayer(att, moe if i % 2 else dense)
+    fan = FanotarConfig(vocab=vocab, width=hidden, norm_eps=1e-6, embedding_scale=float(hidden) ** 0.5,
+                        layers=tuple(fan_layer(i) for i in range(layers)))
+    prompt_len = args.context
+    bench = DesignBench(vocab, prompt_len)
+    whole_engine, timed, context = bench.whole_engine, bench.timed, bench.context
+    dev = lambda v: torch.tensor(v, dtype=torch.int32, device="cuda")
+    bf = torch.bfloat16
 
     def kernel_pairs() -> dict:
         pairs = {}
@@ -592,6 +625,216 @@ def fanotar(args) -> int:
                          "rugezen_ff": 3 * inter // 2, "fanotar_dense_ff": inter, "fanotar_experts": experts, "fanotar_top": top,
                          "fanotar_expert_ff": eff, "fanotar_shared_ff": sff, "fanotar_window": window, "fanotar_conv_taps": taps,
                          "fanotar_layers": "dense and routed feed-forward in turn; every fourth layer reads the cache of the one before",
+                         "vocab": vocab, "context": prompt_len, "dtype": "bf16",
+                         "data": "synthetic uniform token ids, random weights"}}
+    print(json.dumps(record))
+    return 0
+
+
+def bafarax(args) -> int:
+    """The Bafarax decoder beside the Fanotar decoder at the layer sizes of `--shape`: whole-engine throughput, and
+    the like kernels of the two side by side. One JSON line."""
+    import torch
+
+    from tinyserve_llm_amd.config.bafarax import (BafaraxAttention, BafaraxConfig, BafaraxDense, BafaraxExperts, BafaraxLatentAttention,
+                                                  BafaraxLayer, BafaraxMLSTM, FrequencyRamp, Rotation)
+    from tinyserve_llm_amd.config.fanotar import FanotarAttention, FanotarConfig, FanotarExperts, FanotarGatedUnit, FanotarLayer
+    from tinyserve_llm_amd.ops import hip
+
+    sizes = SHAPES[args.shape]
+    sh = sizes["shape"]
+    layers = args.layers or sizes["layers_full"]
+    hidden, nh, nkv, hd, inter, vocab = (sh["hidden_size"], sh["num_attention_heads"], sh["num_key_value_heads"], sh["head_dim"],
+                                         sh["intermediate_size"], sh["vocab_size"])
+    window, taps, experts, top = 1024, 4, 16, 4
+    eff, sff = inter // 8, inter // 2
+    # Bafarax: chunks as long as Fanotar's window; a latent of 256 with 32 turning dimensions beside heads of the shape's
+    # size; a matrix memory of 8 heads whose values are twice as wide as its keys; four ungated experts of 3/8 of the dense
+    # width each (two matrices where a gated unit has three): one dense width per token
+    chunk, rank, q_rank, rot, bff = 1024, 256, 768, 32, 3 * inter // 8
+    mh, md, mv = 8, hidden // 16, hidden // 8
+    b_att = BafaraxAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, scale=hd ** -0.5, rot=Rotation(hd, 250000.0), chunk=chunk)
+    b_lat = BafaraxLatentAttention(heads=nh, dim=hd, rot_dim=rot, vdim=hd, kv_rank=rank, q_rank=q_rank, scale=(hd + rot) ** -0.5,
+                                   rot=Rotation(rot, 10000.0, FrequencyRamp(factor=8.0, original=4096.0, fast=32.0, slow=1.0)), window=window)
+    b_mem = BafaraxMLSTM(heads=mh, dim=md, vdim=mv, gate_cap=15.0)
+    b_moe, b_dense = BafaraxExperts(experts=experts, top=top, ff=bff), BafaraxDense(inter)
+    cycle = (("attention", b_att, b_dense), ("latent_attention", b_lat, b_moe), ("mlstm", b_mem, b_dense), ("latent_attention", b_lat, b_moe))
+    baf = BafaraxConfig(vocab=vocab, width=hidden, norm_eps=1e-6, embedding_scale=float(hidden) ** 0.5,
+                        layers=tuple(BafaraxLayer(*cycle[i % 4]) for i in range(layers)))
+
+    def fan_layer(i):
+        att = FanotarAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, conv=taps, window=window, scale=hd ** -0.5, q_temp_coef=0.1,
+                               q_temp_every=1024, kv_from=i - 1 if i % 4 == 3 else None)
+        moe = FanotarExperts(experts=experts, top=top, scale=2.5, expert=FanotarGatedUnit(eff, 7.0), shared=FanotarGatedUnit(sff, 7.0))
+        return FanotarLayer(att, moe if i % 2 else FanotarGatedUnit(inter, 7.0))
+    fan = FanotarConfig(vocab=vocab, width=hidden, norm_eps=1e-6, embedding_scale=float(hidden) ** 0.5,
+                        layers=tuple(fan_layer(i) for i in range(layers)))
+    prompt_len = args.context
+    bench = DesignBench(vocab, prompt_len)
+    timed, context = bench.timed, bench.context
+    bf = torch.bfloat16
+
+    def kernel_pairs() -> dict:
+        pairs = {}
+        pool_page = 32
+        peaks = hip.measure_peaks()
+        read_peak, mfma_peak, vector_peak = peaks["read_GBps"] * 1e9, peaks["mfma_bf16_TFLOPs"] * 1e12, PEAK_FLOPS["fp32"]
+        slopes = torch.tensor([2.0 ** (-8.0 * (h + 1) / nh) for h in range(nh)], device="cuda")
+        sinks = torch.randn(nh, device="cuda")
+        row = rank + rot
+        # (the decoded tokens stand in the middle of a chunk)
+        for label, starts, counts in (("prompt portion", [0], [prompt_len]), ("decoded tokens, batch 64", [prompt_len + chunk // 2 - 1] * 64, [1] * 64)):
+            ctx, slots, pages = context(starts, counts, pool_page)
+            T, prompt = ctx.num_tokens, ctx.num_tokens > 64
+            of_peak = lambda flops, nbytes, us: ({"frac_of_mfma": flops / us * 1e6 / mfma_peak} if prompt else
+                                                 {"frac_of_read": nbytes / us * 1e6 / read_peak})
+            k = torch.randn(pages, nkv, pool_page, hd, device="cuda").to(bf).permute(0, 2, 1, 3)
+            v = torch.randn(pages, nkv, hd, pool_page, device="cuda").to(bf).permute(0, 3, 1, 2)
+            q = torch.randn(T, nh, hd, device="cuda").to(bf)
+            gate = torch.randn(T, nh * hd, device="cuda")
+            spans = list(zip(starts, counts))
+            seen_w = sum(min(p + 1, window) for s0, n in spans for p in range(s0, s0 + n))
+            seen_c = sum(p % chunk + 1 for s0, n in spans for p in range(s0, s0 + n))
+            # attention over the keys of the position's chunk with learned sinks, against a window, sinks, slopes and a gate
+            us_f = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, window, sinks=sinks, slopes=slopes, gate=gate))
+            us_b = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, 0, sinks=sinks, chunk_mask=chunk))
+            pairs[f"attention in chunks, {label}"] = {
+                "fanotar_us": us_f, "bafarax_us": us_b, "fanotar_keys": seen_w, "bafarax_keys": seen_c,
+                "fanotar": of_peak(4 * nh * hd * seen_w, seen_w * 2 * nkv * hd * 2, us_f),
+                "bafarax": of_peak(4 * nh * hd * seen_c, seen_c * 2 * nkv * hd * 2, us_b)}
+            # attention through the latent: the keys' up-projection on the query's side, the turn of the queries' rotated
+            # part, multi-query attention over the cached rows, the values' up-projection with the gate
+            cache = torch.randn(pages, pool_page, 1, row, device="cuda").to(bf)
+            values = cache[:, :, :, :rank].permute(0, 2, 3, 1).contiguous().permute(0, 3, 1, 2)      # transposed inside a page
+            q32 = torch.randn(T, nh, hd + rot, device="cuda")
+            uk = (torch.randn(nh, hd, rank, device="cuda") * 0.05).to(bf)
+            uv = (torch.randn(nh, hd, rank, device="cuda") * 0.05).to(bf)
+            freqs = torch.rand(rot // 2, dtype=torch.float64, device="cuda")
+            absorbed = torch.empty(T, nh, row, device="cuda")
+            heads = torch.empty(T, nh, hd, dtype=bf, device="cuda")
+
+            def before():
+                hip.heads_gemm(q32[:, :, :hd], uk, absorbed[:, :, :rank])
+                hip.rotate_heads(absorbed[:, :, rank:], q32[:, :, hd:], freqs, 1.2, ctx.positions, interleaved=True)
+            before()
+            attend = lambda: hip.paged_attention_latent(absorbed, cache, rank, ctx, 0, (hd + rot) ** -0.5, window, 0, out_dtype=bf, v_cache=values)
+            mixed = attend()
+            us_before = timed(before)
+            us_att = timed(attend)
+            us_after = timed(lambda: hip.heads_gemm(mixed, uv.transpose(1, 2), heads, gate=gate))
+            flops_att = 2 * nh * seen_w * (row + rank)
+            bytes_att = seen_w * (row + rank) * 2
+            flops_heads = 2 * T * nh * hd * rank
+            pairs[f"attention through a latent, {label}"] = {
+                "fanotar_us": us_f, "bafarax_us": us_before + us_att + us_after, "bafarax_attention_us": us_att,
+                "bafarax_products_before_us": us_before, "bafarax_product_after_us": us_after,
+                "fanotar": of_peak(4 * nh * hd * seen_w, seen_w * 2 * nkv * hd * 2, us_f),
+                "bafarax_attention": of_peak(flops_att, bytes_att, us_att),
+                "bafarax_products": of_peak(2 * flops_heads, 2 * nh * hd * rank * 2 + T * nh * (row + rank) * 4, us_before + us_after)}
+            # between projection and cache: a norm over the whole q and the whole k projection and the rotation; the latents'
+            # norms and the shared key part's rotation; against the convolution, two head norms and its state
+            qkv_row = (nh + 2 * nkv) * hd
+            qkv32 = torch.randn(T, qkv_row + nh * hd, device="cuda")
+            plain32 = qkv32[:, :qkv_row].contiguous()
+            conv = torch.randn(qkv_row, taps, device="cuda")
+            state = torch.zeros(len(starts), taps - 1, qkv_row, device="cuda")
+            nw, qw, kw = torch.ones(hd, device="cuda"), torch.ones(nh * hd, device="cuda"), torch.ones(nkv * hd, device="cuda")
+            rfreqs = torch.rand(hd // 2, dtype=torch.float64, device="cuda")
+
+            def fan_finish():
+                fused = hip.conv_moves_state(ctx)
+                out = hip.conv_finish(qkv32, conv, state, ctx, slots, k, v, nh, nkv, hd, hd, bf, q_norm=nw, k_norm=nw, eps=1e-5,
+                                      temp_coef=0.1, temp_every=1024, moves_state=fused)
+                if not fused:
+                    hip.conv_state_update(state, qkv32, ctx)
+                return out
+
+            def baf_finish():
+                hip.segment_rmsnorm(plain32, 0, nh * hd, qw, 1e-6, out=plain32[:, :nh * hd])
+                hip.segment_rmsnorm(plain32, nh * hd, nkv * hd, kw, 1e-6, out=plain32[:, nh * hd:(nh + nkv) * hd])
+                return hip.qkv_finish(plain32, rfreqs, ctx.positions, slots, k, v, nh, nkv, hd, hd, bf, interleaved=False)
+            down = torch.randn(T, q_rank + row + nh * hd, device="cuda")
+            lqw, lcw = torch.ones(q_rank, device="cuda"), torch.ones(rank, device="cuda")
+            us_f, us_b = timed(fan_finish), timed(baf_finish)
+            us_l = timed(lambda: hip.latent_finish(down, 0, q_rank, q_rank, rank, rot, lqw, lcw, 1e-6, freqs, 1.2, ctx.positions, slots, cache, bf,
+                                                   v_cache=values))
+            nbytes, lbytes = T * qkv_row * (4 + 2), T * ((q_rank + row) * (4 + 2) + rank * 2)
+            pairs[f"between projection and cache, {label}"] = {
+                "fanotar_us": us_f, "bafarax_us": us_b, "bafarax_latent_us": us_l, "bytes": nbytes, "bafarax_latent_bytes": lbytes,
+                "fanotar_frac_of_read": nbytes / us_f * 1e6 / read_peak, "bafarax_frac_of_read": nbytes / us_b * 1e6 / read_peak,
+                "bafarax_latent_frac_of_read": lbytes / us_l * 1e6 / read_peak}
+            # the stream's sum and the norm that reads it, twice a layer in both
+            x32, a32 = torch.randn(T, hidden, device="cuda"), torch.randn(T, hidden, device="cuda")
+            dyt = (torch.full((1,), 0.5, device="cuda"), torch.ones(hidden, device="cuda"), torch.zeros(hidden, device="cuda"))
+            w32 = torch.ones(hidden, device="cuda")
+            us_f = timed(lambda: hip.dyt_stream(x32, a32, dyt, dyt, bf))
+            us_b = timed(lambda: hip.stream_update_norm(x32, a32, None, None, 1.0, (w32, None), 1e-6, out_dtype=bf))
+            sbytes = T * hidden * (3 * 4 + 2)
+            pairs[f"stream sum and norm, {label}"] = {"fanotar_us": us_f, "bafarax_us": us_b, "bytes": sbytes,
+                                                      "fanotar_frac_of_read": sbytes / us_f * 1e6 / read_peak,
+                                                      "bafarax_frac_of_read": sbytes / us_b * 1e6 / read_peak}
+            # the experts: two products of ungated experts with a squared relu, against three of gated ones, equal work
+            x16 = torch.randn(T, hidden, device="cuda").to(bf)
+            router, corr = torch.randn(experts, hidden, device="cuda") * 0.02, torch.zeros(experts, device="cuda")
+            wgu = (torch.randn(experts, 2 * eff, hidden, device="cuda") * 0.02).to(bf)
+            wd = (torch.randn(experts, hidden, eff, device="cuda") * 0.02).to(bf)
+            wup = (torch.randn(experts, bff, hidden, device="cuda") * 0.02).to(bf)
+            wdn = (torch.randn(experts, hidden, bff, device="cuda") * 0.02).to(bf)
+            ids, wts = hip.moe_route(x16, router, None, top, 1.0, True, softmax_chosen=True)
+            tr_f, tr_b = hip.moe_tile_rows(ids.numel(), experts, bf, (hidden, eff)), hip.moe_tile_rows(ids.numel(), experts, bf, (hidden, bff))
+            g_f, g_b = hip.moe_group(ids, experts, tr_f), hip.moe_group(ids, experts, tr_b)
+            us_route_f = timed(lambda: hip.moe_route(x16, router, corr, top, 2.5))
+            us_route_b = timed(lambda: hip.moe_route(x16, router, None, top, 1.0, True, softmax_chosen=True))
+
+            def fan_products():
+                unit = hip.moe_gemm(x16, wgu, g_f, bf, per_token=True, glu=(7.0, 1.702, 1.0))
+                return hip.moe_combine(hip.moe_gemm(unit, wd, g_f, torch.float32, per_token=False), wts)
+
+            def baf_products():
+                act = hip.moe_gemm(x16, wup, g_b, bf, per_token=True, activation="relu2")
+                return hip.moe_combine(hip.moe_gemm(act, wdn, g_b, torch.float32, per_token=False), wts)
+            us_f, us_b = timed(fan_products), timed(baf_products)
+            flops_f, flops_b = 2 * T * top * 3 * eff * hidden, 2 * T * top * 2 * bff * hidden
+            touched_f, touched_b = min(experts, T * top) * 3 * eff * hidden * 2, min(experts, T * top) * 2 * bff * hidden * 2
+            pairs[f"experts' products, {label}"] = {"fanotar_us": us_f, "bafarax_us": us_b, "fanotar_routing_us": us_route_f,
+                                                    "bafarax_routing_us": us_route_b, "fanotar": of_peak(flops_f, touched_f, us_f),
+                                                    "bafarax": of_peak(flops_b, touched_b, us_b)}
+            # the matrix memory: the scan and what follows it; beside it the engine's other recurrence, a minGRU of the model's
+            # width (a number per channel where this one keeps a matrix per head)
+            width = 2 * mh * md + mh * mv + 2 * mh + mh * mv
+            proj = torch.randn(T, width, device="cuda")
+            gb = torch.zeros(2 * mh, device="cuda")
+            mstate = torch.zeros(len(starts), hip.mlstm_state_size(mh, md, mv), device="cuda")
+            mw = torch.ones(mh * mv, device="cuda")
+
+            def memory():
+                o = hip.mlstm_scan(proj, gb[:mh], gb[mh:], mstate, ctx.cu_seqlens, ctx.state_slots, mh, md, mv, 15.0)
+                return hip.mlstm_finish(o, mw, proj[:, width - mh * mv:], mh, mv, 1e-6, bf)
+            us_b = timed(memory)
+            us_scan = timed(lambda: hip.mlstm_scan(proj, gb[:mh], gb[mh:], mstate, ctx.cu_seqlens, ctx.state_slots, mh, md, mv, 15.0))
+            zxg = torch.randn(T, 3 * hidden, device="cuda")
+            gstate = torch.zeros(len(starts), hidden, device="cuda")
+            us_g = timed(lambda: hip.mingru_scan(zxg, None, gstate, ctx.cu_seqlens, ctx.state_slots, max(counts), bf))
+            mbytes = T * width * 4 + T * mh * mv * (4 + 4 + 2) + 2 * len(starts) * mstate.shape[1] * 4
+            gbytes = T * hidden * (3 * 4 + 2) + 2 * len(starts) * hidden * 4
+            mflops = 4 * T * mh * md * mv
+            pairs[f"matrix memory, {label}"] = {"bafarax_us": us_b, "bafarax_scan_us": us_scan, "rugezen_mingru_us": us_g,
+                                                "bafarax_bytes": mbytes, "rugezen_mingru_bytes": gbytes, "bafarax_flops_fp32": mflops,
+                                                "bafarax_frac_of_read": mbytes / us_b * 1e6 / read_peak,
+                                                "bafarax_frac_of_fp32_vector": mflops / us_b * 1e6 / vector_peak,
+                                                "rugezen_mingru_frac_of_read": gbytes / us_g * 1e6 / read_peak}
+        pairs["peaks"] = {"read_GBps": read_peak / 1e9, "mfma_bf16_TFLOPs": mfma_peak / 1e12, "fp32_vector_TFLOPs_published": vector_peak / 1e12}
+        return pairs
+
+    record = {"designs": {} if args.kernels_only else {"fanotar": bench.whole_engine(fan), "bafarax": bench.whole_engine(baf)},
+              "kernels": kernel_pairs(),
+              "config": {"shape": args.shape, "layers": layers, "hidden": hidden, "heads": nh, "kv_heads": nkv, "head_dim": hd,
+                         "fanotar_window": window, "fanotar_experts": experts, "fanotar_top": top, "fanotar_expert_ff": eff,
+                         "fanotar_shared_ff": sff, "bafarax_chunk": chunk, "bafarax_window": window, "bafarax_kv_rank": rank,
+                         "bafarax_q_rank": q_rank, "bafarax_rot_dim": rot, "bafarax_expert_ff": bff,
+                         "bafarax_memory": {"heads": mh, "dim": md, "vdim": mv},
+                         "bafarax_layers": "in turn: attention in chunks with a dense feed-forward, latent attention with experts, "
+                                           "a matrix memory with a dense feed-forward, latent attention with experts",
                          "vocab": vocab, "context": prompt_len, "dtype": "bf16",
                          "data": "synthetic uniform token ids, random weights"}}
     print(json.dumps(record))
@@ -728,6 +971,10 @@ def main() -> int:
     ap.add_argument("--fanotar", action="store_true",
                     help="measure the Fanotar decoder beside the Rugezen decoder at the layer sizes of --shape: whole-engine "
                          "throughput and the like kernels side by side; one JSON line")
+    ap.add_argument("--bafarax", action="store_true",
+                    help="measure the Bafarax decoder beside the Fanotar decoder at the layer sizes of --shape: whole-engine "
+                         "throughput and the like kernels side by side; one JSON line")
+    ap.add_argument("--kernels-only", action="store_true", help="with --bafarax: the kernels side by side, no whole-engine runs")
     ap.add_argument("--kernel-classes", action="store_true",
                     help="time one decode step's kernels class by class (bytes, microseconds, GB/s) and exit")
     ap.add_argument("--peaks", action="store_true",
@@ -755,6 +1002,8 @@ def main() -> int:
         return designs(args)
     if args.fanotar:
         return fanotar(args)
+    if args.bafarax:
+        return bafarax(args)
     sizes = SHAPES[args.shape]
     full_layers = sizes["layers_full"]
     args.layers = args.layers or full_layers

@@ -76,10 +76,10 @@ def test_plans_of_layers_that_run_with_another_layers_weights():
     assert [r.layer for r in model.spec.order] == [0, 1, 2, 2, 1, 3] and len(model.layers) == 4
     assert all(r.cache is None and r.store for r in model.spec.order), "every run keeps a cache or state of its own"
     plan = model.cache_plan()
-    # chunks of one position; the latent's rows (latent and shared key part, no separate values) for its window, once per
-    # run; and a layer that sees everything
+    # chunks of one position; the latent's rows (latent and shared key part; the latent once more as the values) for its
+    # window, once per run; and a layer that sees everything
     assert [(e.owner, e.kv.window, e.kv.num_kv_heads, e.kv.head_dim, e.kv.v_dim) for e in plan] == \
-        [(0, 1, 2, 16, 16), (1, 70, 1, 32, 0), (4, 70, 1, 32, 0), (5, 0, 1, 8, 24)]
+        [(0, 1, 2, 16, 16), (1, 70, 1, 32, 16), (4, 70, 1, 32, 16), (5, 0, 1, 8, 24)]
     # per head S [dim, vdim], n [dim] and m, for each of the two runs
     assert [(e.run, tuple(e.state.shape)) for e in model.state_plan()] == [(2, (16 * 16 + 16 + 1,)), (3, (16 * 16 + 16 + 1,))]
     assert model.graph_safe()

@@ -217,11 +217,12 @@ def test_latent_norms_shared_key_part_and_cache_rows(dtype, sizes):
     down = torch.randn(len(positions), q_rank + rank + rot + extra) * 2
     wq, wc = 1 + 0.1 * torch.randn(q_rank), 1 + 0.1 * torch.randn(rank)
     cache = torch.zeros(6, page, 1, rank + rot, dtype=dtype, device=DEV)
+    values = torch.zeros(6, 1, rank, page, dtype=dtype, device=DEV).permute(0, 3, 1, 2)      # transposed inside a page
     slots = [3 * page + 1, 0, 5 * page + 15, 17, 2 * page, 4 * page + 7, 4 * page + 8]
     dev = lambda t: torch.tensor(t, dtype=torch.int32, device=DEV)
     d = down.to(DEV)
     cq = h.latent_finish(d, 0, q_rank, q_rank, rank, rot, wq.to(DEV), wc.to(DEV), 1e-5, freqs.to(DEV) if rot else None, amp,
-                         dev(positions), dev(slots), cache, dtype)
+                         dev(positions), dev(slots), cache, dtype, v_cache=values)
     r = down.to(F64)
     tol = dict(atol=2e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=3e-2, rtol=1e-2)
     torch.testing.assert_close(cq.cpu().to(F64), plain.unit_rms(r[:, :q_rank], 1e-5) * wq.to(F64), **tol)
@@ -229,6 +230,8 @@ def test_latent_norms_shared_key_part_and_cache_rows(dtype, sizes):
     kr = plain.rotate(r[:, q_rank + rank:q_rank + rank + rot], torch.tensor(positions), freqs if rot else torch.zeros(0, dtype=F64), amp, True)
     for i, s in enumerate(slots):
         torch.testing.assert_close(cache[s // page, s % page, 0].cpu().to(F64), torch.cat([c[i], kr[i]]), **tol)
+        assert torch.equal(values[s // page, s % page, 0], cache[s // page, s % page, 0, :rank]), "the values are the latent once more"
+    assert int((values != 0).any(-1).sum()) == len(slots), "no other slot was written"
     assert torch.equal(d.cpu(), down), "the projected rows stay as they were (the gate is read from them later)"
 
 
@@ -267,7 +270,7 @@ def test_products_per_head_as_stored_and_transposed_with_a_gate(dtype, sizes):
     torch.testing.assert_close(y.cpu().to(F64), want, **tol)
 
 
-def latent_case(dtype, H, rank, rot, page, length, queries, stand_out, scale, window, seed=0, portion_from=None):
+def latent_case(dtype, H, rank, rot, page, length, queries, stand_out, scale, window, seed=0, portion_from=None, mfma=None):
     """Cached rows [c | r] of one request on shuffled pages; queries as in `chunk_case`. The key that stands out has its
     whole row along the query's direction. The oracle sees one key/value head: keys the rows, values their first `rank`."""
     h = hip()
@@ -286,15 +289,20 @@ def latent_case(dtype, H, rank, rot, page, length, queries, stand_out, scale, wi
     pages = -(-length // page)
     table = torch.randperm(pages + 3, generator=gen)[:pages].tolist()
     cache = torch.zeros(pages + 3, page, 1, row, dtype=dtype, device=DEV)
+    values = torch.zeros(pages + 3, 1, rank, page, dtype=dtype, device=DEV).permute(0, 3, 1, 2)
     rr = rows64.to(dtype)
     at = torch.arange(length)
-    cache[torch.tensor(table)[at // page].to(DEV), (at % page).to(DEV), 0] = rr.to(DEV)
+    pg, off = torch.tensor(table)[at // page].to(DEV), (at % page).to(DEV)
+    cache[pg, off, 0] = rr.to(DEV)
+    values[pg, off, 0] = rr[:, :rank].to(DEV)
     q = q64.float().to(DEV)                                                 # (queries stay 32-bit up to the scores)
     if portion_from is None:
         ctx = step_context([table] * len(queries), page, queries, [1] * len(queries))
     else:
         ctx = step_context([table], page, [portion_from], [len(queries)])
-    out = h.paged_attention_latent(q, cache, rank, ctx, 0, scale, window, 0, out_dtype=dtype)
+    out = h.paged_attention_latent(q, cache, rank, ctx, 0, scale, window, 0, out_dtype=dtype, v_cache=values)
+    if mfma is not None:
+        assert h.latent_mfma_takes(q, cache, values, rank) == mfma, "the case was made for the other kernel"
     keys = rr.to(F64)
     want = plain.masked_attention(q.cpu().to(F64), keys[:, None, :], keys[:, None, :rank], torch.tensor(queries), scale,
                                   "window" if window else "full", window, None)
@@ -303,10 +311,15 @@ def latent_case(dtype, H, rank, rot, page, length, queries, stand_out, scale, wi
 
 @pytest.mark.parametrize("form", sorted(FORMS))
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("window, sizes", [(1, (3, 40, 8)), (7, (3, 34, 6)), (16, (2, 16, 16)), (50, (3, 40, 8)), (64, (4, 128, 16)),
-                                           (70, (2, 16, 16)), (96, (4, 128, 16)), (130, (8, 256, 32)), (257, (2, 512, 64)), (65, (4, 64, 0))])
-def test_latent_attention_window_edges(dtype, window, sizes, form):
-    (H, rank, rot), page = sizes, 16
+@pytest.mark.parametrize("page", [16, 32])
+@pytest.mark.parametrize("window, sizes", [(1, (3, 40, 8)), (7, (3, 34, 6)), (16, (2, 16, 16)), (50, (3, 48, 8)), (64, (4, 128, 16)),
+                                           (70, (5, 16, 16)), (96, (4, 128, 16)), (130, (8, 256, 32)), (257, (2, 512, 64)), (65, (4, 64, 0)),
+                                           (33, (24, 32, 8)), (100, (32, 256, 64)), (31, (16, 80, 24))])
+def test_latent_attention_window_edges(dtype, window, sizes, form, page):
+    """Pages of 16 keys go to the kernel that is 32-bit throughout, as float32 always does; pages of 32 in bfloat16 go to
+    the matrix cores where the sizes allow: tokens of fewer than 16 heads share a tile, heads beyond 16 take a second one."""
+    H, rank, rot = sizes
+    mfma = dtype == torch.bfloat16 and page == 32 and rank % 16 == 0 and rot % 8 == 0 and rank <= 256 and rank + rot <= 320
     if window > 100:
         length = 4 * window + 15
         inside = {q: q - window + 1 for q in (window - 1, 3 * window + 9)}
@@ -317,7 +330,7 @@ def test_latent_attention_window_edges(dtype, window, sizes, form):
         outside = {q: q - window for q in (200, 599)}
     queries = sorted({0, 127, 128, 129, *inside, *outside})
     out, want, v, queries = latent_case(dtype, H, rank, rot, page, length, queries, {**inside, **outside}, (rank + rot) ** -0.5,
-                                        window, portion_from=FORMS[form])
+                                        window, portion_from=FORMS[form], mfma=mfma)
     torch.testing.assert_close(out, want, **tolerance(dtype))
     for q, key in inside.items():
         if q in queries:
@@ -329,12 +342,13 @@ def test_latent_attention_window_edges(dtype, window, sizes, form):
 
 @pytest.mark.parametrize("form", sorted(FORMS))
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(3, 40, 8), (2, 16, 16), (8, 256, 32), (5, 34, 6)])
-def test_latent_attention_far_keys_and_page_borders(dtype, sizes, form):
+@pytest.mark.parametrize("page", [16, 32])
+@pytest.mark.parametrize("sizes", [(3, 48, 8), (2, 16, 16), (8, 256, 32), (5, 34, 6), (20, 128, 16)])
+def test_latent_attention_far_keys_and_page_borders(dtype, sizes, form, page):
     H, rank, rot = sizes
-    stand_out = {699: 3, 650: 15, 651: 16, 652: 17, 653: 653, 500: 255, 501: 256, 31: 0}
-    queries = [0, 1, 2, 3, 15, 16, 17, 31, 500, 501, 650, 651, 652, 653, 699]
-    out, want, v, qs = latent_case(dtype, H, rank, rot, 16, 700, queries, stand_out, (rank + rot) ** -0.5, 0, portion_from=FORMS[form])
+    stand_out = {699: 3, 650: 15, 651: 16, 652: 17, 653: 653, 500: 255, 501: 256, 31: 0, 32: 31, 33: 32}
+    queries = [0, 1, 2, 3, 15, 16, 17, 31, 32, 33, 500, 501, 650, 651, 652, 653, 699]
+    out, want, v, qs = latent_case(dtype, H, rank, rot, page, 700, queries, stand_out, (rank + rot) ** -0.5, 0, portion_from=FORMS[form])
     torch.testing.assert_close(out, want, **tolerance(dtype))
     assert decides(want[qs.index(699), 0], v[3]), "the far key decides the row"
 

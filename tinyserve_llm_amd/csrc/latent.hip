@@ -6,7 +6,8 @@
 //     weight, 32-bit, to a place and storage type of its own (norms over whole projections or parts of them).
 //   * `ts_latent_finish`: what lies between the fused down-projection and the cache: the query latent's norm, the
 //     key/value latent's norm, the rotation of the shared key part (pairs (2i, 2i+1), angle in 64-bit, cosine and
-//     sine times an amplitude), and the write of [c | r] to the token's cache slot.
+//     sine times an amplitude), and the write of [c | r] to the token's cache slot (and of c once more into the
+//     pages that hold the values transposed, for the matrix-core kernel of latent_mfma.hip).
 //   * `ts_rotate_heads`: a stretch of every head turned by the token's position, to a place of its own.
 //   * `ts_heads_gemm`: y[t, h, :] = x[t, h, :] . W[h] for per-head matrices with free strides (so W may be used as
 //     stored or transposed), 32-bit multiply-adds in ascending k; optionally times sigmoid(gate) on the way out.
@@ -72,7 +73,7 @@ latent_finish_kernel(TO* __restrict__ cq_out, TO* __restrict__ cache, const floa
                      int q_off, int q_rank, int kv_off, int rank, int rot, const float* __restrict__ q_weight,
                      const float* __restrict__ kv_weight, float eps, const double* __restrict__ freqs, float amplitude,
                      const int32_t* __restrict__ positions, const int32_t* __restrict__ slots, int page_size, int64_t kp,
-                     int64_t ks) {
+                     int64_t ks, TO* __restrict__ vcache, int64_t vp, int64_t vd) {
   __shared__ float red[LT_WAVES];
   const int t = blockIdx.x;
   const float* row = down + (int64_t)t * stride;
@@ -91,7 +92,12 @@ latent_finish_kernel(TO* __restrict__ cq_out, TO* __restrict__ cache, const floa
   float squares = 0.f;
   for (int d = threadIdx.x; d < rank; d += LT_THREADS) squares = fmaf(c[d], c[d], squares);
   const float inv = 1.0f / sqrtf(lt_block_sum(squares, red) / (float)rank + eps);
-  for (int d = threadIdx.x; d < rank; d += LT_THREADS) Num<TO>::st(dst + d, c[d] * inv * kv_weight[d]);
+  TO* vdst = vcache ? vcache + page * vp + off : nullptr;  // the latent once more, transposed inside the page
+  for (int d = threadIdx.x; d < rank; d += LT_THREADS) {
+    const float v = c[d] * inv * kv_weight[d];
+    Num<TO>::st(dst + d, v);
+    if (vdst) Num<TO>::st(vdst + (int64_t)d * vd, v);
+  }
   const int pos = positions[t];
   for (int pair = threadIdx.x; pair < rot / 2; pair += LT_THREADS) {
     float cs, sn;
@@ -105,15 +111,15 @@ latent_finish_kernel(TO* __restrict__ cq_out, TO* __restrict__ cache, const floa
 extern "C" int ts_latent_finish(void* cq_out, void* cache, int out_dtype, const float* down, int64_t stride, int q_off,
                                 int q_rank, int kv_off, int rank, int rot, const float* q_weight, const float* kv_weight,
                                 float eps, const double* freqs, float amplitude, const int32_t* positions,
-                                const int32_t* slots, int page_size, int64_t kp, int64_t ks, int num_tokens,
-                                hipStream_t stream) {
+                                const int32_t* slots, int page_size, int64_t kp, int64_t ks, void* vcache, int64_t vp,
+                                int64_t vd, int num_tokens, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
   if (rank <= 0 || rot < 0 || rot % 2 || q_rank < 0 || q_off < 0 || kv_off < 0 || page_size <= 0 ||
       q_off + q_rank > stride || kv_off + rank + rot > stride || (rot > 0 && !freqs))
     return TS_BAD_SHAPE;
 #define LT_FINISH(TO) \
   latent_finish_kernel<TO><<<num_tokens, LT_THREADS, 0, stream>>>((TO*)cq_out, (TO*)cache, down, stride, q_off, q_rank, kv_off, \
-      rank, rot, q_weight, kv_weight, eps, freqs, amplitude, positions, slots, page_size, kp, ks)
+      rank, rot, q_weight, kv_weight, eps, freqs, amplitude, positions, slots, page_size, kp, ks, (TO*)vcache, vp, vd)
   if (out_dtype == 0) LT_FINISH(float);
   else if (out_dtype == 1) LT_FINISH(bf16_t);
   else return TS_BAD_DTYPE;

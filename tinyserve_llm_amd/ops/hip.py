@@ -97,7 +97,9 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_moe_group": [p, p, p, i, i, i, i, p],
         "ts_moe_gemm": [p, i, p, i, p, p, p, i, i, i, i, i, i, f, f, f, i, p],
         "ts_segment_rmsnorm": [p, i, i64, p, i64, i, p, f, i, p],
-        "ts_latent_finish": [p, p, i, p, i64, i, i, i, i, i, p, p, f, p, f, p, p, i, i64, i64, i, p],
+        "ts_latent_finish": [p, p, i, p, i64, i, i, i, i, i, p, p, f, p, f, p, p, i, i64, i64, p, i64, i64, i, p],
+        "ts_latent_mfma_takes": [i, i],
+        "ts_paged_attention_latent_mfma": [p, i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i, f, i, i, p],
         "ts_rotate_heads": [p, i, i64, i64, p, i64, i64, i, i, i, p, f, p, i, p],
         "ts_heads_gemm": [p, i, i64, i64, p, i, i64, i64, p, i, i64, i64, i64, i, i, i, i, p, i64, p],
         "ts_paged_attention_latent": [p, i, p, i, p, i, p, p, p, i, i, i, i, i, i64, i64, i, f, i, i, p],
@@ -2119,12 +2121,14 @@ LATENT_MAX_ROW = 640       # and of a cached row (latent and shared rotated key 
 
 def latent_finish(down: torch.Tensor, q_off: int, q_rank: int, kv_off: int, rank: int, rot: int, q_weight: torch.Tensor | None,
                   kv_weight: torch.Tensor, eps: float, freqs: torch.Tensor | None, amplitude: float, positions: torch.Tensor,
-                  slots: torch.Tensor | None, cache: torch.Tensor | None, out_dtype: torch.dtype) -> torch.Tensor | None:
+                  slots: torch.Tensor | None, cache: torch.Tensor | None, out_dtype: torch.dtype,
+                  v_cache: torch.Tensor | None = None) -> torch.Tensor | None:
     """From the fused down-projection's rows (float32) to the query latent and the cache. Columns [q_off, + q_rank):
     divided by their root mean square times `q_weight`, returned as [tokens, q_rank] of `out_dtype` (None if q_rank is
     0). Columns [kv_off, + rank): likewise with `kv_weight`, the latent c; the next `rot` columns turn by the position
-    (pairs (2i, 2i+1), cosine and sine times `amplitude`); [c | turned] goes to the token's slot of `cache`."""
-    _gpu(down, q_weight, kv_weight, freqs, positions, slots, cache)
+    (pairs (2i, 2i+1), cosine and sine times `amplitude`); [c | turned] goes to the token's slot of `cache`, and c
+    once more to the token's slot of `v_cache` (a view [pages, page_size, 1, rank], in memory transposed inside a page)."""
+    _gpu(down, q_weight, kv_weight, freqs, positions, slots, cache, v_cache)
     T = down.shape[0]
     _need(down.dtype == torch.float32 and down.dim() == 2 and down.is_contiguous(), "the projected rows must be contiguous float32")
     _need(q_rank == 0 or (q_weight is not None and q_weight.dtype == torch.float32 and q_weight.shape == (q_rank,) and q_weight.is_contiguous()),
@@ -2133,15 +2137,21 @@ def latent_finish(down: torch.Tensor, q_off: int, q_rank: int, kv_off: int, rank
     _need(0 <= q_off and q_off + q_rank <= down.shape[1] and 0 <= kv_off and kv_off + rank + rot <= down.shape[1], "the stretches lie inside a row")
     _check_freqs(freqs, rot)
     _check_step_vectors(T, positions=positions, slots=slots)
-    page_size, kp, ks = 1, 0, 0
+    page_size, kp, ks, vp, vd = 1, 0, 0, 0, 0
     if cache is not None:
         _need(slots is not None, "a cache write needs the slots")
         _check_latent_cache(cache, rank + rot, out_dtype)
         page_size, kp, ks = cache.shape[1], cache.stride(0), cache.stride(1)
+    if v_cache is not None:
+        _need(cache is not None and v_cache.dtype == out_dtype and v_cache.dim() == 4 and v_cache.shape[:3] == cache.shape[:3]
+              and v_cache.shape[3] == rank and v_cache.stride(1) == 1,
+              lambda: f"the values' view must be [pages, page_size, 1, {rank}] like the rows', slots side by side in memory")
+        vp, vd = v_cache.stride(0), v_cache.stride(3)
     cq = torch.empty((T, q_rank), dtype=out_dtype, device=down.device) if q_rank else None
     _run("latent_finish", library().ts_latent_finish(
         _ptr(cq), _ptr(cache), _code(out_dtype), _ptr(down), down.shape[1], q_off, q_rank, kv_off, rank, rot, _ptr(q_weight),
-        _ptr(kv_weight), float(eps), _ptr(freqs), float(amplitude), _ptr(positions), _ptr(slots), page_size, kp, ks, T, _stream()))
+        _ptr(kv_weight), float(eps), _ptr(freqs), float(amplitude), _ptr(positions), _ptr(slots), page_size, kp, ks,
+        _ptr(v_cache), vp, vd, T, _stream()))
     return cq
 
 
@@ -2178,12 +2188,26 @@ def heads_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: torch.
     return out
 
 
+def latent_mfma_takes(q: torch.Tensor, cache: torch.Tensor, v_cache: torch.Tensor | None, rank: int) -> bool:
+    """Whether the matrix-core kernel serves these operands (else the one-workgroup-per-token kernel does): bfloat16
+    caches in pages of 32 keys with the values once more in transposed pages, 32-bit queries, rows and ranks of the
+    sizes it is built for."""
+    return (v_cache is not None and q.dtype == torch.float32 and cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
+            and cache.shape[1] == 32 and v_cache.stride(1) == 1 and bool(library().ts_latent_mfma_takes(rank, q.shape[2]))
+            and all(st % 8 == 0 for st in (cache.stride(0), cache.stride(1), v_cache.stride(0), v_cache.stride(3)))
+            and cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0)
+
+
 def paged_attention_latent(q: torch.Tensor, cache: torch.Tensor, rank: int, ctx, space: int, scale: float, window: int = 0,
-                           chunk_mask: int = 0, out_dtype: torch.dtype | None = None) -> torch.Tensor:
+                           chunk_mask: int = 0, out_dtype: torch.dtype | None = None, v_cache: torch.Tensor | None = None
+                           ) -> torch.Tensor:
     """Multi-query attention of a packed step over cached rows [c | r] (c the first `rank` numbers, which are also
     the values): q [tokens, heads, rank + rot] (float32, or the cache's type), out [tokens, heads, rank] = the softmax
-    weights' sum of c. Causal, with a sliding `window` or chunks (`chunk_mask`) as `paged_attention` has them."""
-    _gpu(q, cache)
+    weights' sum of c. Causal, with a sliding `window` or chunks (`chunk_mask`) as `paged_attention` has them. With
+    `v_cache` (the values once more, [pages, page_size, 1, rank], transposed inside a page) bfloat16 caches of the
+    sizes it serves go to the matrix-core kernel; everything else, float32 always, to a kernel that is 32-bit
+    throughout and whose sums depend on the token's position alone."""
+    _gpu(q, cache, v_cache)
     _need(chunk_mask >= 0 and window >= 0 and not (chunk_mask and window), "a sliding window or chunks, both counted in positions")
     T, H, row = q.shape
     _need(q.is_contiguous() and 0 < rank <= min(row, LATENT_MAX_RANK) and row <= LATENT_MAX_ROW,
@@ -2195,10 +2219,29 @@ def paged_attention_latent(q: torch.Tensor, cache: torch.Tensor, rank: int, ctx,
     _need(tables.dtype == torch.int32 and tables.dim() == 2 and tables.is_contiguous(), "block_tables must be contiguous int32 [requests, pages]")
     _check_step_vectors(T, seq_of_token=ctx.seq_of_token, positions=ctx.positions)
     out = torch.empty((T, H, rank), dtype=out_dtype or cache.dtype, device=q.device)
+    mask = -chunk_mask if chunk_mask else int(window)
+    if latent_mfma_takes(q, cache, v_cache, rank) and out.dtype in (torch.float32, torch.bfloat16):
+        _need(v_cache.shape == (*cache.shape[:3], rank), "the values' view must match the rows'")
+        tile_tokens = max(1, 16 // H)
+        tiles, num_tiles = None, T
+        if ctx.max_query_len > 1 and tile_tokens > 1:
+            # (a token with 16 heads or more is a tile of its own: no list; else tiles of several tokens of one request)
+            tiles = ctx.scratch.get(("latent_tiles", tile_tokens))
+            if tiles is None:
+                flat = attention_tiles(ctx.host_cu_seqlens, ctx.host_starts, tile_tokens)
+                tiles = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(q.device, non_blocking=True)
+                ctx.scratch[("latent_tiles", tile_tokens)] = tiles
+            num_tiles = tiles.shape[0]
+        _run("paged_attention_latent_mfma", library().ts_paged_attention_latent_mfma(
+            _ptr(out), _code(out.dtype), _ptr(q), _ptr(cache), _ptr(v_cache), _ptr(tables), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
+            _ptr(tiles), num_tiles, tile_tokens if tiles is not None else 1, T, H, rank, row - rank, cache.shape[1], cache.stride(0),
+            cache.stride(1), v_cache.stride(0), v_cache.stride(3), v_cache.stride(1), tables.shape[1], float(scale), mask,
+            _page_run(table_page // cache.shape[1]), _stream()))
+        return out
     _run("paged_attention_latent", library().ts_paged_attention_latent(
         _ptr(out), _code(out.dtype), _ptr(q), _code(q.dtype), _ptr(cache), _code(cache.dtype), _ptr(tables), _ptr(ctx.seq_of_token),
         _ptr(ctx.positions), T, H, rank, row - rank, cache.shape[1], cache.stride(0), cache.stride(1), tables.shape[1], float(scale),
-        -chunk_mask if chunk_mask else int(window), _page_run(table_page // cache.shape[1]), _stream()))
+        mask, _page_run(table_page // cache.shape[1]), _stream()))
     return out
 
 

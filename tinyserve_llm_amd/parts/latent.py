@@ -1,7 +1,7 @@
 """Attention through a low-rank latent. A token's keys and values of all heads are up-projections of one latent c
 (`kv_rank` numbers, divided by its root mean square and weighted), and every head's key has a further part of
 `rot_dim` rotated dimensions that all heads share; queries come through a latent of their own (`q_rank`). Only
-[c | rotated part] is cached, one row per token. The up-projections move to the query's and the output's side:
+[c | rotated part] is cached, one row per token (and c once more, in the pages that hold values transposed). The up-projections move to the query's and the output's side:
     score_h(i, j) = ((W_uk,h^T q_h,plain) . c_j + q_h,rot . r_j) * scale,   out_h = W_uv,h (sum_j p_j c_j),
 so attention runs as multi-query attention over the cached rows, whose first `kv_rank` numbers are also the values
 (`hip.paged_attention_latent`), with a product per head before it and one after it (`hip.heads_gemm`). A sliding
@@ -70,8 +70,9 @@ class LatentAttention(Mixer):
         return max(self.q_rank + self.row_size + self.out_size, 2 * self.num_heads * self.row_size)
 
     def kv_spec(self) -> KVSpec:
-        # one row per token, no separate values: they are the row's first kv_rank numbers
-        return KVSpec(1, self.row_size, self.window or self.chunk, 0)
+        # one row per token; its first kv_rank numbers are the values, which the cache keeps once more in the pages that
+        # hold values transposed, for the matrix-core kernel
+        return KVSpec(1, self.row_size, self.window or self.chunk, self.kv_rank)
 
     def keep_streaming_copies(self) -> int:
         self.down_packed, self.uq_packed, self.o_packed = streaming_copy(self.down), streaming_copy(self.uq), streaming_copy(self.o)
@@ -84,16 +85,17 @@ class LatentAttention(Mixer):
         if enc is not None and not getattr(enc, "interleaved", True):
             raise ValueError("the latent's rotated part pairs dimensions (2i, 2i + 1)")
         down = linear(x, self.down, out_dtype=torch.float32, packed=self.down_packed)
-        slots, cache = (ctx.slot_mapping[mem.space], mem.k_cache) if mem.store else (None, None)
+        slots, cache, values = (ctx.slot_mapping[mem.space], mem.k_cache, mem.v_cache) if mem.store else (None, None, None)
         cq = hip.latent_finish(down, 0, self.q_rank, self.q_rank, C, R, self.q_norm, self.kv_norm, self.norm_eps, freqs, amplitude,
-                               ctx.positions, slots, cache, x.dtype)
+                               ctx.positions, slots, cache, x.dtype, v_cache=values)
         q = linear(cq, self.uq, out_dtype=torch.float32, packed=self.uq_packed).view(T, H, D + R)
         # the keys' up-projection on the query's side: W_uk,h^T q_h beside the turned part, in the cached row's order
         absorbed = torch.empty((T, H, C + R), dtype=torch.float32, device=x.device)
         hip.heads_gemm(q[:, :, :D], self.uk.view(H, D, C), absorbed[:, :, :C])
         if R:
             hip.rotate_heads(absorbed[:, :, C:], q[:, :, D:], freqs, amplitude, ctx.positions, interleaved=True)
-        mixed = hip.paged_attention_latent(absorbed, mem.k_cache, C, ctx, mem.space, self.scale, self.window, self.chunk, out_dtype=x.dtype)
+        mixed = hip.paged_attention_latent(absorbed, mem.k_cache, C, ctx, mem.space, self.scale, self.window, self.chunk, out_dtype=x.dtype,
+                                           v_cache=mem.v_cache)
         # the values' up-projection on the output's side, the gate on its way out
         heads = torch.empty((T, H, V), dtype=x.dtype, device=x.device)
         hip.heads_gemm(mixed, self.uv.view(H, V, C).transpose(1, 2), heads,
