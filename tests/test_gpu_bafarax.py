@@ -370,15 +370,18 @@ def mlstm_weights(H, D, V, cap):
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("sizes", [(3, 20, 28, 8.0), (1, 16, 16, 15.0), (2, 18, 270, 5.0), (4, 64, 128, 12.0), (2, 32, 48, 12.0),
                                    (1, 1, 1, 2.0), (2, 128, 64, 6.0), (1, 300, 20, 4.0)])
-def test_matrix_memory_over_steps_slots_and_gates_at_their_caps(dtype, sizes):
+@pytest.mark.parametrize("portions", [[1, 2, 13, 1, 5, 31, 3], [1, 2, 13, 1, 5, 64, 3], [200, 1, 32]])
+def test_matrix_memory_over_steps_slots_and_gates_at_their_caps(dtype, sizes, portions):
     """Three requests of unequal length in packed steps of changing portions (one token, two, many), each with its state in
     a slot of its own among slots that hold another request's leftovers until they are cleared; gate sums far beyond the
-    cap on either side; heads whose values span several workgroups, and heads of one dimension."""
+    cap on either side; heads whose values span several workgroups, and heads of one dimension. Steps in which every
+    request feeds few tokens walk token by token; a step in which one feeds 32 or more is worked in chunks of 64 (whole
+    chunks, a chunk's rest, single tokens of other requests beside them)."""
     h = hip()
     H, D, V, cap = sizes
     W, m, width = mlstm_weights(H, D, V, cap)
     gen = torch.Generator().manual_seed(H * 1000 + D)
-    lengths = [37, 1, 90]
+    lengths = [37, 1, 90] if portions[0] < 100 else [150, 1, 333]
     bi, bf = torch.randn(H, generator=gen), torch.randn(H, generator=gen) + 1
     W["i.b"], W["f.b"] = bi.to(F64), bf.to(F64)
     norm_w = 1 + 0.1 * torch.randn(H * V, generator=gen)
@@ -399,14 +402,14 @@ def test_matrix_memory_over_steps_slots_and_gates_at_their_caps(dtype, sizes):
     slots = [4, 0, 2]
     state[slots] = 0.0                                                      # (what the manager does when it hands a slot out)
     cursors, got, tick = [0, 0, 0], [[], [], []], 0
-    portions = [1, 2, 13, 1, 5, 64, 3]
     while any(c < n for c, n in zip(cursors, lengths)):
         live = [i for i in range(3) if cursors[i] < lengths[i]]
         counts = [min(portions[(tick + 2 * i) % len(portions)], lengths[i] - cursors[i]) for i in live]
         tick += 1
         proj = torch.cat([rows[i][cursors[i]:cursors[i] + n] for i, n in zip(live, counts)]).to(DEV)
         cu = torch.tensor([0] + list(itertools.accumulate(counts)), dtype=torch.int32, device=DEV)
-        o = h.mlstm_scan(proj, bi.to(DEV), bf.to(DEV), state, cu, torch.tensor([slots[i] for i in live], dtype=torch.int32, device=DEV), H, D, V, cap)
+        o = h.mlstm_scan(proj, bi.to(DEV), bf.to(DEV), state, cu, torch.tensor([slots[i] for i in live], dtype=torch.int32, device=DEV), H, D, V, cap,
+                         host_cu_seqlens=[0] + list(itertools.accumulate(counts)))
         y = h.mlstm_finish(o, norm_w.to(DEV), proj[:, gates_at + 2 * H:], H, V, 1e-5, dtype)
         at = 0
         for i, n in zip(live, counts):

@@ -104,6 +104,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_heads_gemm": [p, i, i64, i64, p, i, i64, i64, p, i, i64, i64, i64, i, i, i, i, p, i64, p],
         "ts_paged_attention_latent": [p, i, p, i, p, i, p, p, p, i, i, i, i, i, i64, i64, i, f, i, i, p],
         "ts_mlstm_scan": [p, p, i64, p, p, p, p, p, i, i, i, i, i, f, f, p],
+        "ts_mlstm_scan_chunks": [p, p, i64, p, p, p, p, p, p, p, p, p, i, i, i, i, i, f, f, p],
         "ts_mlstm_finish": [p, i, p, p, p, i64, i, i, i, f, p],
         "ts_moe_combine": [p, p, p, p, i, i, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
@@ -2265,12 +2266,33 @@ def mlstm_state_size(heads: int, dim: int, vdim: int) -> int:
     return heads * (dim * vdim + dim + 1)
 
 
+MLSTM_CHUNK = 64           # tokens of a chunk of the chunked form,
+MLSTM_CHUNKS_FROM = 32     # which serves steps in which some request feeds at least this many tokens
+
+
+def mlstm_chunks(host_cu_seqlens: list[int]) -> tuple[list[int], list[int]]:
+    """The chunks of a packed step for the chunked scan: ([(first token, tokens, request, 1 if the request's last)...]
+    flattened, [first chunk of each request..., number of chunks])."""
+    flat: list[int] = []
+    cu = [0]
+    for s in range(len(host_cu_seqlens) - 1):
+        a, b = host_cu_seqlens[s], host_cu_seqlens[s + 1]
+        for t in range(a, b, MLSTM_CHUNK):
+            flat += (t, min(MLSTM_CHUNK, b - t), s, int(t + MLSTM_CHUNK >= b))
+        cu.append(len(flat) // 4)
+    return flat, cu
+
+
 def mlstm_scan(proj: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, state: torch.Tensor, cu_seqlens: torch.Tensor,
-               state_slots: torch.Tensor, heads: int, dim: int, vdim: int, cap: float) -> torch.Tensor:
+               state_slots: torch.Tensor, heads: int, dim: int, vdim: int, cap: float, host_cu_seqlens: list[int] | None = None,
+               scratch: dict | None = None) -> torch.Tensor:
     """The recurrence over a packed step. proj float32 [tokens, >= 2 heads dim + heads vdim + 2 heads]: per token
     q | k | v | the input gates' sums | the forget gates' sums (then whatever else the fused projection makes); state
     float32 [slots, heads (dim vdim + dim + 1)], read at each request's slot and written back. Returns o float32
-    [tokens, heads vdim], before the heads' norm."""
+    [tokens, heads vdim], before the heads' norm. With `host_cu_seqlens` (the step's lengths on the host) a step in which
+    some request feeds `MLSTM_CHUNKS_FROM` tokens or more is worked in chunks of `MLSTM_CHUNK` tokens: products over a
+    chunk's tokens and a short scan over the chunks instead of a walk token by token (`scratch`: the step's, to keep the
+    chunk list for the model's other layers)."""
     _gpu(proj, i_bias, f_bias, state, cu_seqlens, state_slots)
     T = proj.shape[0]
     need = 2 * heads * dim + heads * vdim + 2 * heads
@@ -2283,6 +2305,23 @@ def mlstm_scan(proj: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, s
     _need(cu_seqlens.dtype == torch.int32 and cu_seqlens.shape == (S + 1,) and state_slots.dtype == torch.int32, "cu_seqlens int32 [requests + 1], slots int32 [requests]")
     _need(0 < dim <= MLSTM_MAX_DIM and cap > 0, lambda: f"heads of up to {MLSTM_MAX_DIM} dimensions, a positive cap")
     out = torch.empty((T, heads * vdim), dtype=torch.float32, device=proj.device)
+    if host_cu_seqlens is not None and max((b - a for a, b in zip(host_cu_seqlens, host_cu_seqlens[1:])), default=0) >= MLSTM_CHUNKS_FROM:
+        _need(len(host_cu_seqlens) == S + 1 and host_cu_seqlens[-1] == T, "the host's lengths are the step's")
+        kept = scratch.get("mlstm_chunks") if scratch is not None else None
+        if kept is None:
+            flat, cu = mlstm_chunks(host_cu_seqlens)
+            kept = (torch.tensor(flat, dtype=torch.int32).view(-1, 4).to(proj.device, non_blocking=True),
+                    torch.tensor(cu, dtype=torch.int32).to(proj.device, non_blocking=True))
+            if scratch is not None:
+                scratch["mlstm_chunks"] = kept
+        chunks, chunk_cu = kept
+        C = chunks.shape[0]
+        buf = torch.empty((C, heads, dim * vdim + dim), dtype=torch.float32, device=proj.device)
+        scalars = torch.empty((C, heads, 3), dtype=torch.float32, device=proj.device)      # (b_L, m_loc), and the m before the chunk
+        _run("mlstm_scan_chunks", library().ts_mlstm_scan_chunks(
+            _ptr(out), _ptr(proj), proj.shape[1], _ptr(i_bias), _ptr(f_bias), _ptr(state), _ptr(chunks), _ptr(chunk_cu), _ptr(state_slots),
+            _ptr(buf), _ptr(scalars), scalars.data_ptr() + 8 * C * heads, C, S, heads, dim, vdim, float(cap), float(dim) ** -0.5, _stream()))
+        return out
     _run("mlstm_scan", library().ts_mlstm_scan(_ptr(out), _ptr(proj), proj.shape[1], _ptr(i_bias), _ptr(f_bias), _ptr(state), _ptr(cu_seqlens),
                                                _ptr(state_slots), S, heads, dim, vdim, mlstm_columns(dim, vdim), float(cap), float(dim) ** -0.5, _stream()))
     return out

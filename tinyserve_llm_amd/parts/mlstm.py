@@ -6,7 +6,8 @@ moves as
     m' = max(f + m, i),  S' = exp(f + m - m') S + exp(i - m') k v^T,  n' = exp(f + m - m') n + exp(i - m') k,
 and reads out o = S'^T q / (max(|n' . q|, exp(-m')) + 1e-6); each head's o is divided by its root mean square, the
 heads side by side are multiplied by a weight and by sigmoid(g), and the output projection follows. S, n and m start at
-zero, are kept in 32-bit floats in the request's state slot, and are carried from step to step (`hip.mlstm_scan`);
+zero, are kept in 32-bit floats in the request's state slot, and are carried from step to step (`hip.mlstm_scan`:
+token by token where every request feeds few tokens, in chunks of 64 tokens where one feeds many);
 gates, exponentials and the heads' norm are 32-bit in every storage type."""
 
 from __future__ import annotations
@@ -59,6 +60,6 @@ class MLSTM(Mixer):
         H = self.num_heads
         proj = linear(x, self.proj, out_dtype=torch.float32, packed=self.proj_packed)
         o = hip.mlstm_scan(proj, self.gate_bias[:H], self.gate_bias[H:], mem.state, ctx.cu_seqlens, ctx.state_slots, H,
-                           self.head_dim, self.value_dim, self.gate_cap)
+                           self.head_dim, self.value_dim, self.gate_cap, host_cu_seqlens=ctx.host_cu_seqlens, scratch=ctx.scratch)
         gated = hip.mlstm_finish(o, self.norm, proj[:, self.gate_at:], H, self.value_dim, self.norm_eps, x.dtype)
         return linear(gated, self.o, out_dtype=torch.float32, packed=self.o_packed)
