@@ -631,19 +631,13 @@ def fanotar(args) -> int:
     return 0
 
 
-def bafarax(args) -> int:
-    """The Bafarax decoder beside the Fanotar decoder at the layer sizes of `--shape`: whole-engine throughput, and
-    the like kernels of the two side by side. One JSON line."""
-    import torch
-
+def bafarax_design(shape: str, layers: int | None):
+    """The Bafarax configuration that `--bafarax` measures at the layer sizes of `shape`, and those sizes by name."""
     from tinyserve_llm_amd.config.bafarax import (BafaraxAttention, BafaraxConfig, BafaraxDense, BafaraxExperts, BafaraxLatentAttention,
                                                   BafaraxLayer, BafaraxMLSTM, FrequencyRamp, Rotation)
-    from tinyserve_llm_amd.config.fanotar import FanotarAttention, FanotarConfig, FanotarExperts, FanotarGatedUnit, FanotarLayer
-    from tinyserve_llm_amd.ops import hip
-
-    sizes = SHAPES[args.shape]
+    sizes = SHAPES[shape]
     sh = sizes["shape"]
-    layers = args.layers or sizes["layers_full"]
+    layers = layers or sizes["layers_full"]
     hidden, nh, nkv, hd, inter, vocab = (sh["hidden_size"], sh["num_attention_heads"], sh["num_key_value_heads"], sh["head_dim"],
                                          sh["intermediate_size"], sh["vocab_size"])
     window, taps, experts, top = 1024, 4, 16, 4
@@ -661,6 +655,23 @@ def bafarax(args) -> int:
     cycle = (("attention", b_att, b_dense), ("latent_attention", b_lat, b_moe), ("mlstm", b_mem, b_dense), ("latent_attention", b_lat, b_moe))
     baf = BafaraxConfig(vocab=vocab, width=hidden, norm_eps=1e-6, embedding_scale=float(hidden) ** 0.5,
                         layers=tuple(BafaraxLayer(*cycle[i % 4]) for i in range(layers)))
+
+    return baf, dict(layers=layers, hidden=hidden, nh=nh, nkv=nkv, hd=hd, inter=inter, vocab=vocab, window=window, taps=taps,
+                     experts=experts, top=top, eff=eff, sff=sff, chunk=chunk, rank=rank, q_rank=q_rank, rot=rot, bff=bff, mh=mh, md=md, mv=mv)
+
+
+def bafarax(args) -> int:
+    """The Bafarax decoder beside the Fanotar decoder at the layer sizes of `--shape`: whole-engine throughput, and
+    the like kernels of the two side by side. One JSON line."""
+    import torch
+
+    from tinyserve_llm_amd.config.fanotar import FanotarAttention, FanotarConfig, FanotarExperts, FanotarGatedUnit, FanotarLayer
+    from tinyserve_llm_amd.ops import hip
+
+    baf, z = bafarax_design(args.shape, args.layers)
+    layers, hidden, nh, nkv, hd, inter, vocab = z["layers"], z["hidden"], z["nh"], z["nkv"], z["hd"], z["inter"], z["vocab"]
+    window, taps, experts, top, eff, sff = z["window"], z["taps"], z["experts"], z["top"], z["eff"], z["sff"]
+    chunk, rank, q_rank, rot, bff, mh, md, mv = z["chunk"], z["rank"], z["q_rank"], z["rot"], z["bff"], z["mh"], z["md"], z["mv"]
 
     def fan_layer(i):
         att = FanotarAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, conv=taps, window=window, scale=hd ** -0.5, q_temp_coef=0.1,
@@ -808,10 +819,12 @@ def bafarax(args) -> int:
             mw = torch.ones(mh * mv, device="cuda")
 
             def memory():
-                o = hip.mlstm_scan(proj, gb[:mh], gb[mh:], mstate, ctx.cu_seqlens, ctx.state_slots, mh, md, mv, 15.0)
+                o = hip.mlstm_scan(proj, gb[:mh], gb[mh:], mstate, ctx.cu_seqlens, ctx.state_slots, mh, md, mv, 15.0,
+                                   host_cu_seqlens=ctx.host_cu_seqlens, scratch=ctx.scratch)
                 return hip.mlstm_finish(o, mw, proj[:, width - mh * mv:], mh, mv, 1e-6, bf)
             us_b = timed(memory)
-            us_scan = timed(lambda: hip.mlstm_scan(proj, gb[:mh], gb[mh:], mstate, ctx.cu_seqlens, ctx.state_slots, mh, md, mv, 15.0))
+            us_scan = timed(lambda: hip.mlstm_scan(proj, gb[:mh], gb[mh:], mstate, ctx.cu_seqlens, ctx.state_slots, mh, md, mv, 15.0,
+                                                   host_cu_seqlens=ctx.host_cu_seqlens, scratch=ctx.scratch))
             zxg = torch.randn(T, 3 * hidden, device="cuda")
             gstate = torch.zeros(len(starts), hidden, device="cuda")
             us_g = timed(lambda: hip.mingru_scan(zxg, None, gstate, ctx.cu_seqlens, ctx.state_slots, max(counts), bf))

@@ -3,8 +3,8 @@
 // more, transposed inside its pages ([rank, page_size]), because the product P.V wants, for one dimension,
 // consecutive keys side by side. All heads of a token share the keys, so the heads are the rows of the matrix
 // products: a workgroup owns a tile of 16 rows (16 heads of one token, or all heads of several tokens of one
-// request where a token has fewer than 16), its four waves walk the tile's keys in 32-key steps, each wave every
-// fourth step, with a running maximum and sum of their own, and add their parts up through shared memory, one wave
+// request where a token has fewer than 16), its four waves (eight where the step has few tiles) walk the tile's keys in
+// 32-key steps, each wave every fourth (eighth) step, with a running maximum and sum of their own, and add their parts up through shared memory, one wave
 // after the other (the order of every sum is fixed).
 //     S^T[key, row] = K[key, :] . Q[row, :]       v_mfma_f32_16x16x32_bf16, keys as rows, Q from shared memory
 //     P = 2^(S scale log2 e - m), 32-bit, carried into the second product as two bfloat16 terms
@@ -13,20 +13,20 @@
 // 32-bit. Causal, with a sliding window or chunks (`ts_first_key`).
 #include "attention_mfma.h"
 
-#define LM_WAVES 4
-#define LM_THREADS (LM_WAVES * TS_WAVE)
 #define LM_ROWS 16
+#define LM_FEW_TILES 512       // fewer workgroups than this: eight waves a tile instead of four
 
 // NKS: 32-wide steps over a cached row that the kernel is built for (row <= 32 NKS); NVB: 16-wide blocks of the
 // values (rank <= 16 NVB). Steps and blocks beyond the actual sizes are skipped by uniform branches.
-template <int NKS, int NVB, typename TO>
-__global__ void __launch_bounds__(LM_THREADS)
+template <int NKS, int NVB, int LM_WAVES, typename TO>
+__global__ void __launch_bounds__(LM_WAVES * TS_WAVE)
 latent_attention_mfma_kernel(TO* __restrict__ out, const float* __restrict__ q, const bf16_t* __restrict__ k_cache,
                              const bf16_t* __restrict__ v_cache, const int32_t* __restrict__ block_tables,
                              const int32_t* __restrict__ seq_of_token, const int32_t* __restrict__ positions,
                              const int32_t* __restrict__ tiles, int num_tiles, int tile_tokens, int nh, int rank, int row,
                              int64_t kp, int64_t ks, int64_t vp, int64_t vd, int max_blocks, float scale_log2, int window,
                              int page_run, int num_tokens) {
+  constexpr int LM_THREADS = LM_WAVES * TS_WAVE;
   constexpr int QS = NKS * 32 + 8;                          // a row of the queries in shared memory, skewed
   __shared__ __attribute__((aligned(16))) bf16_t q_s[LM_ROWS][QS];
   __shared__ __attribute__((aligned(16))) float o_s[LM_ROWS][NVB * 16 + 4];
@@ -72,17 +72,18 @@ latent_attention_mfma_kernel(TO* __restrict__ out, const float* __restrict__ q, 
     const int64_t page = ((int64_t)table[pg >> page_run] << page_run) + (pg & ((1 << page_run) - 1));
     const bf16_t* kbase = k_cache + page * kp;
     const bf16_t* vbase = v_cache + page * vp;
+    // every lane loads, whatever its step and block, from an address inside the page (the row's last piece, the last
+    // dimension's keys): loads under branches would be waited for one by one. What is read past the row's end meets
+    // zeros of the queries; blocks past the values' end are not multiplied.
     uint4 kf[2][NKS], vf[NVB];
 #pragma unroll
-    for (int tau = 0; tau < 2; ++tau)
+    for (int tau = 0; tau < 2; ++tau) {
+      const bf16_t* krow = kbase + (int64_t)(8 * (r >> 2) + 4 * tau + (r & 3)) * ks;
 #pragma unroll
-      for (int c = 0; c < NKS; ++c) {
-        const int key = 8 * (r >> 2) + 4 * tau + (r & 3), d = 32 * c + 8 * g;
-        kf[tau][c] = (c < nks && d < row) ? *(const uint4*)(kbase + (int64_t)key * ks + d) : make_uint4(0, 0, 0, 0);
-      }
+      for (int c = 0; c < NKS; ++c) kf[tau][c] = *(const uint4*)(krow + min(32 * c + 8 * g, row - 8));
+    }
 #pragma unroll
-    for (int db = 0; db < NVB; ++db)
-      vf[db] = db < nvb ? *(const uint4*)(vbase + (int64_t)(16 * db + r) * vd + 8 * g) : make_uint4(0, 0, 0, 0);
+    for (int db = 0; db < NVB; ++db) vf[db] = *(const uint4*)(vbase + (int64_t)min(16 * db + r, rank - 1) * vd + 8 * g);
     float s[8];
 #pragma unroll
     for (int tau = 0; tau < 2; ++tau) {
@@ -155,7 +156,9 @@ latent_attention_mfma_kernel(TO* __restrict__ out, const float* __restrict__ q, 
     const int rr = i / rank, d = i - rr * rank;
     const int tok = rr / heads_here, head = 16 * hb + rr % heads_here;
     if (tok >= count || tok >= tile_tokens) continue;
-    const float total = l_s[0][rr] + l_s[1][rr] + l_s[2][rr] + l_s[3][rr];
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < LM_WAVES; ++w) total += l_s[w][rr];
     Num<TO>::st(out + ((int64_t)(t0 + tok) * nh + head) * rank + d, o_s[rr][d] / total);
   }
 }
@@ -181,19 +184,23 @@ extern "C" int ts_paged_attention_latent_mfma(void* out, int out_dtype, const fl
     return TS_BAD_SHAPE;
   dim3 grid(((num_tiles + 7) / 8) * 8, (nh + 15) / 16);
   const float scale_log2 = scale * 1.4426950408889634f;
+  const bool few = (int64_t)grid.x * grid.y < LM_FEW_TILES;
 #define LM_LAUNCH(NKS, NVB, TO) \
-  latent_attention_mfma_kernel<NKS, NVB, TO><<<grid, LM_THREADS, 0, stream>>>((TO*)out, q, (const bf16_t*)k_cache, \
+  if (few) LM_LAUNCH_W(NKS, NVB, 8, TO); else LM_LAUNCH_W(NKS, NVB, 4, TO)
+#define LM_LAUNCH_W(NKS, NVB, W, TO) \
+  latent_attention_mfma_kernel<NKS, NVB, W, TO><<<grid, W * TS_WAVE, 0, stream>>>((TO*)out, q, (const bf16_t*)k_cache, \
       (const bf16_t*)v_cache, block_tables, seq_of_token, positions, tiles, num_tiles, tile_tokens, nh, rank, row, kp, ks, vp, vd, \
       max_blocks, scale_log2, window, page_run, num_tokens)
 #define LM_PICK(TO) \
   do { \
-    if (row <= 160 && rank <= 128) LM_LAUNCH(5, 8, TO); \
-    else LM_LAUNCH(10, 16, TO); \
+    if (row <= 160 && rank <= 128) { LM_LAUNCH(5, 8, TO); } \
+    else { LM_LAUNCH(10, 16, TO); } \
   } while (0)
   if (out_dtype == 0) LM_PICK(float);
   else if (out_dtype == 1) LM_PICK(bf16_t);
   else return TS_BAD_DTYPE;
 #undef LM_PICK
 #undef LM_LAUNCH
+#undef LM_LAUNCH_W
   return ts_check_launch();
 }

@@ -2229,6 +2229,7 @@ def paged_attention_latent(q: torch.Tensor, cache: torch.Tensor, rank: int, ctx,
             # (a token with 16 heads or more is a tile of its own: no list; else tiles of several tokens of one request)
             tiles = ctx.scratch.get(("latent_tiles", tile_tokens))
             if tiles is None:
+                _need(not torch.cuda.is_current_stream_capturing(), "the tile list is made before a graph is recorded")
                 flat = attention_tiles(ctx.host_cu_seqlens, ctx.host_starts, tile_tokens)
                 tiles = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(q.device, non_blocking=True)
                 ctx.scratch[("latent_tiles", tile_tokens)] = tiles
@@ -2309,6 +2310,8 @@ def mlstm_scan(proj: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, s
         _need(len(host_cu_seqlens) == S + 1 and host_cu_seqlens[-1] == T, "the host's lengths are the step's")
         kept = scratch.get("mlstm_chunks") if scratch is not None else None
         if kept is None:
+            # (a list copied from the host while a graph is being recorded would be read again, from memory long freed, at every replay)
+            _need(not torch.cuda.is_current_stream_capturing(), "the chunk list is made before a graph is recorded: pass the step's scratch")
             flat, cu = mlstm_chunks(host_cu_seqlens)
             kept = (torch.tensor(flat, dtype=torch.int32).view(-1, 4).to(proj.device, non_blocking=True),
                     torch.tensor(cu, dtype=torch.int32).to(proj.device, non_blocking=True))
