@@ -314,12 +314,13 @@ def latent_case(dtype, H, rank, rot, page, length, queries, stand_out, scale, wi
 @pytest.mark.parametrize("page", [16, 32])
 @pytest.mark.parametrize("window, sizes", [(1, (3, 40, 8)), (7, (3, 34, 6)), (16, (2, 16, 16)), (50, (3, 48, 8)), (64, (4, 128, 16)),
                                            (70, (5, 16, 16)), (96, (4, 128, 16)), (130, (8, 256, 32)), (257, (2, 512, 64)), (65, (4, 64, 0)),
-                                           (33, (24, 32, 8)), (100, (32, 256, 64)), (31, (16, 80, 24))])
+                                           (33, (24, 32, 8)), (100, (32, 256, 64)), (31, (16, 80, 24)), (200, (40, 64, 8))])
 def test_latent_attention_window_edges(dtype, window, sizes, form, page):
     """Pages of 16 keys go to the kernel that is 32-bit throughout, as float32 always does; pages of 32 in bfloat16 go to
-    the matrix cores where the sizes allow: tokens of fewer than 16 heads share a tile, heads beyond 16 take a second one."""
+    the matrix cores where the sizes allow: tokens of fewer than 32 heads share a tile, heads beyond 32 take a second one;
+    steps of few tiles cut a tile's keys into stretches that a second kernel adds up."""
     H, rank, rot = sizes
-    mfma = dtype == torch.bfloat16 and page == 32 and rank % 16 == 0 and rot % 8 == 0 and rank <= 256 and rank + rot <= 320
+    mfma = dtype == torch.bfloat16 and page == 32 and rank % 16 == 0 and rot % 8 == 0
     if window > 100:
         length = 4 * window + 15
         inside = {q: q - window + 1 for q in (window - 1, 3 * window + 9)}

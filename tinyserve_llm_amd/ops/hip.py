@@ -99,7 +99,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_segment_rmsnorm": [p, i, i64, p, i64, i, p, f, i, p],
         "ts_latent_finish": [p, p, i, p, i64, i, i, i, i, i, p, p, f, p, f, p, p, i, i64, i64, p, i64, i64, i, p],
         "ts_latent_mfma_takes": [i, i],
-        "ts_paged_attention_latent_mfma": [p, i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i, f, i, i, p],
+        "ts_paged_attention_latent_mfma": [p, i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i, f, i, i, i, p, p, p],
         "ts_rotate_heads": [p, i, i64, i64, p, i64, i64, i, i, i, p, f, p, i, p],
         "ts_heads_gemm": [p, i, i64, i64, p, i, i64, i64, p, i, i64, i64, i64, i, i, i, i, p, i64, p],
         "ts_paged_attention_latent": [p, i, p, i, p, i, p, p, p, i, i, i, i, i, i64, i64, i, f, i, i, p],
@@ -2189,6 +2189,11 @@ def heads_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: torch.
     return out
 
 
+LATENT_TILE_ROWS = 32     # rows (token, head) of a workgroup of the matrix-core kernel
+LATENT_MAX_SPLITS = 16    # stretches a tile's keys may be cut into,
+LATENT_FEW_GROUPS = 512   # where the step has fewer workgroups than half of this
+
+
 def latent_mfma_takes(q: torch.Tensor, cache: torch.Tensor, v_cache: torch.Tensor | None, rank: int) -> bool:
     """Whether the matrix-core kernel serves these operands (else the one-workgroup-per-token kernel does): bfloat16
     caches in pages of 32 keys with the values once more in transposed pages, 32-bit queries, rows and ranks of the
@@ -2223,10 +2228,10 @@ def paged_attention_latent(q: torch.Tensor, cache: torch.Tensor, rank: int, ctx,
     mask = -chunk_mask if chunk_mask else int(window)
     if latent_mfma_takes(q, cache, v_cache, rank) and out.dtype in (torch.float32, torch.bfloat16):
         _need(v_cache.shape == (*cache.shape[:3], rank), "the values' view must match the rows'")
-        tile_tokens = max(1, 16 // H)
+        tile_tokens = max(1, LATENT_TILE_ROWS // H)
         tiles, num_tiles = None, T
         if ctx.max_query_len > 1 and tile_tokens > 1:
-            # (a token with 16 heads or more is a tile of its own: no list; else tiles of several tokens of one request)
+            # (a token with 32 heads or more is a tile of its own: no list; else tiles of several tokens of one request)
             tiles = ctx.scratch.get(("latent_tiles", tile_tokens))
             if tiles is None:
                 _need(not torch.cuda.is_current_stream_capturing(), "the tile list is made before a graph is recorded")
@@ -2234,11 +2239,18 @@ def paged_attention_latent(q: torch.Tensor, cache: torch.Tensor, rank: int, ctx,
                 tiles = torch.tensor(flat, dtype=torch.int32).view(-1, 2).to(q.device, non_blocking=True)
                 ctx.scratch[("latent_tiles", tile_tokens)] = tiles
             num_tiles = tiles.shape[0]
+        # few tiles (decoded tokens): a tile's keys in stretches, a workgroup each, and a second kernel that adds them up
+        groups = num_tiles * -(-H // LATENT_TILE_ROWS)
+        capacity = tables.shape[1] * table_page
+        steps = -(-(min(window + 32, capacity) if window > 0 else min(chunk_mask, capacity) if chunk_mask else capacity) // 32)
+        splits = max(1, min(LATENT_MAX_SPLITS, LATENT_FEW_GROUPS // groups, steps // 2)) if groups < LATENT_FEW_GROUPS // 2 else 1
+        part_o = torch.empty((T, H, splits, rank), dtype=torch.float32, device=q.device) if splits > 1 else None
+        part_ml = torch.empty((T, H, splits, 2), dtype=torch.float32, device=q.device) if splits > 1 else None
         _run("paged_attention_latent_mfma", library().ts_paged_attention_latent_mfma(
             _ptr(out), _code(out.dtype), _ptr(q), _ptr(cache), _ptr(v_cache), _ptr(tables), _ptr(ctx.seq_of_token), _ptr(ctx.positions),
             _ptr(tiles), num_tiles, tile_tokens if tiles is not None else 1, T, H, rank, row - rank, cache.shape[1], cache.stride(0),
             cache.stride(1), v_cache.stride(0), v_cache.stride(3), v_cache.stride(1), tables.shape[1], float(scale), mask,
-            _page_run(table_page // cache.shape[1]), _stream()))
+            _page_run(table_page // cache.shape[1]), splits, _ptr(part_o), _ptr(part_ml), _stream()))
         return out
     _run("paged_attention_latent", library().ts_paged_attention_latent(
         _ptr(out), _code(out.dtype), _ptr(q), _code(q.dtype), _ptr(cache), _code(cache.dtype), _ptr(tables), _ptr(ctx.seq_of_token),
