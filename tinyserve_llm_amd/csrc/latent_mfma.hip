@@ -61,13 +61,33 @@ latent_attention_mfma_kernel(TO* __restrict__ out, float* __restrict__ part_o, f
   const int lo_min = ts_first_key(pos0, window), pos_max = pos0 + count - 1;
   const int32_t* table = block_tables + (int64_t)seq_of_token[t0] * max_blocks;
 
-  // the tile's queries, rounded once, zeros where there is no row or no dimension
-  for (int i = threadIdx.x; i < LM_ROWS * CPW * 128; i += LM_THREADS) {
-    const int rr = i / (CPW * 128), d = i - rr * (CPW * 128);
-    const int tok = rr / heads_here, head = heads_block * hb + rr % heads_here;
-    float v = 0.f;
-    if (tok < count && tok < tile_tokens && d < row) v = q[((int64_t)(t0 + tok) * nh + head) * row + d];
-    q_s[rr][d] = f2bf(v);
+  // the tile's queries, rounded once, zeros where there is no row or no dimension. Every thread's loads go out
+  // together, each from an address inside the step's queries (a row without a token reads the tile's first).
+  __shared__ int64_t src_s[LM_ROWS];
+  if (threadIdx.x < LM_ROWS) {
+    const int tok = threadIdx.x / heads_here, head = heads_block * hb + threadIdx.x % heads_here;
+    src_s[threadIdx.x] = (tok < count && tok < tile_tokens) ? ((int64_t)(t0 + tok) * nh + head) * row : -1;
+  }
+  __syncthreads();
+  {
+    constexpr int F4 = CPW * 32, PER = LM_ROWS * F4 / LM_THREADS;       // 16-byte pieces of a row; of a thread
+    const int64_t fallback = ((int64_t)t0 * nh + heads_block * hb) * row;
+    float4 got[PER];
+#pragma unroll
+    for (int it = 0; it < PER; ++it) {
+      const int i = threadIdx.x + it * LM_THREADS, rr = i / F4, d = 4 * (i - rr * F4);
+      const int64_t src = src_s[rr];
+      got[it] = *(const float4*)(q + (src < 0 ? fallback : src) + min(d, row - 4));
+    }
+#pragma unroll
+    for (int it = 0; it < PER; ++it) {
+      const int i = threadIdx.x + it * LM_THREADS, rr = i / F4, d = 4 * (i - rr * F4);
+      const bool in = src_s[rr] >= 0 && d < row;
+      uint2 packed;
+      packed.x = in ? pack_bf16(got[it].x, got[it].y) : 0u;
+      packed.y = in ? pack_bf16(got[it].z, got[it].w) : 0u;
+      *(uint2*)&q_s[rr][d] = packed;
+    }
   }
   __syncthreads();
 
@@ -222,29 +242,34 @@ latent_attention_mfma_kernel(TO* __restrict__ out, float* __restrict__ part_o, f
   }
 }
 
-// One wave per (token, head): the stretches' parts to one row. m is in units of log2.
+// One workgroup per (token, head), a thread per value column: the stretches' parts to one row. m is in units of log2.
 template <typename TO>
 __global__ void __launch_bounds__(LM_THREADS)
 latent_attention_combine_kernel(TO* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml,
-                                int rank, int splits, int64_t items) {
-  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
-  const int64_t item = (int64_t)blockIdx.x * LM_WAVES + wave;
-  if (item >= items) return;
+                                int rank, int splits) {
+  const int64_t item = blockIdx.x;
   const float* ml = part_ml + item * splits * 2;
-  float top = -INFINITY;
-  for (int z = 0; z < splits; ++z) top = fmaxf(top, ml[2 * z]);
+  float ms[LM_MAX_SPLITS], ls[LM_MAX_SPLITS], top = -INFINITY;
+#pragma unroll
+  for (int z = 0; z < LM_MAX_SPLITS; ++z) {
+    ms[z] = ml[2 * min(z, splits - 1)];
+    ls[z] = ml[2 * min(z, splits - 1) + 1];
+    top = fmaxf(top, ms[z]);
+  }
   float weight[LM_MAX_SPLITS], total = 0.f;
 #pragma unroll
   for (int z = 0; z < LM_MAX_SPLITS; ++z) {
-    weight[z] = z < splits ? fast_exp2(ml[2 * z] - top) : 0.f;   // (a stretch without keys: 2^-inf = 0)
-    if (z < splits) total += weight[z] * ml[2 * z + 1];
+    weight[z] = z < splits ? fast_exp2(ms[z] - top) : 0.f;   // (a stretch without keys: 2^-inf = 0)
+    total += weight[z] * ls[z];
   }
   const float inv = 1.0f / total;
-  for (int d = lane; d < rank; d += TS_WAVE) {
+  for (int d = threadIdx.x; d < rank; d += LM_THREADS) {
+    float part[LM_MAX_SPLITS];
+#pragma unroll
+    for (int z = 0; z < LM_MAX_SPLITS; ++z) part[z] = part_o[(item * splits + min(z, splits - 1)) * rank + d];
     float sum = 0.f;
 #pragma unroll
-    for (int z = 0; z < LM_MAX_SPLITS; ++z)
-      if (z < splits) sum = fmaf(weight[z], part_o[(item * splits + z) * rank + d], sum);
+    for (int z = 0; z < LM_MAX_SPLITS; ++z) sum = fmaf(weight[z], part[z], sum);
     Num<TO>::st(out + item * rank + d, sum * inv);
   }
 }
@@ -285,8 +310,7 @@ extern "C" int ts_paged_attention_latent_mfma(void* out, int out_dtype, const fl
     else LM_LAUNCH(5, 8, TO); \
     if (splits > 1) { \
       const int64_t items = (int64_t)num_tokens * nh; \
-      latent_attention_combine_kernel<TO><<<(unsigned)((items + LM_WAVES - 1) / LM_WAVES), LM_THREADS, 0, stream>>>( \
-          (TO*)out, part_o, part_ml, rank, splits, items); \
+      latent_attention_combine_kernel<TO><<<(unsigned)items, LM_THREADS, 0, stream>>>((TO*)out, part_o, part_ml, rank, splits); \
     } \
   } while (0)
   if (out_dtype == 0) LM_PICK(float);

@@ -90,11 +90,11 @@ stream_update_norm_kernel(float* __restrict__ x, const void* __restrict__ a, int
 // or on whether an operand is there stands between two loads: an operand that is not there is read from another of
 // its shape and counts times 0), and the updated row stays in registers between the sum of squares and the scaling.
 #define RS_HELD 16
-template <typename H, int HELD, bool NORMS>
+template <typename H, typename W, int HELD, bool NORMS>
 __global__ void __launch_bounds__(RS_THREADS)
 stream_update_norm_held_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ b,
                                const H* __restrict__ bias, float mult, H* __restrict__ h1, H* __restrict__ h2,
-                               const H* __restrict__ w1, const H* __restrict__ w2, float eps,
+                               const W* __restrict__ w1, const W* __restrict__ w2, float eps,
                                const int32_t* __restrict__ rows, int width) {
   __shared__ float scratch[RS_THREADS / TS_WAVE];
   const int64_t r = blockIdx.x;
@@ -104,9 +104,9 @@ stream_update_norm_held_kernel(float* __restrict__ x, const float* __restrict__ 
   // an operand that is not there is read from another of its size (the row itself; a norm's weight) and not used
   const float* ar = (a ? a : x) + t * width;
   const float* br = (b ? b : x) + t * width;
-  const H* wa = w1 ? w1 : w2;
-  const H* wb = w2 ? w2 : w1;
-  const H* bs = bias ? bias : (NORMS ? wa : (const H*)xr);
+  const W* wa = w1 ? w1 : w2;
+  const W* wb = w2 ? w2 : w1;
+  const H* bs = bias ? bias : (NORMS ? (const H*)wa : (const H*)xr);
   float v[HELD], va[HELD], vb[HELD], vbias[HELD], wva[HELD], wvb[HELD];
 #pragma unroll
   for (int j = 0; j < HELD; ++j) {
@@ -116,8 +116,8 @@ stream_update_norm_held_kernel(float* __restrict__ x, const float* __restrict__ 
     vb[j] = br[i];
     vbias[j] = Num<H>::ld(bs + i);
     if constexpr (NORMS) {
-      wva[j] = Num<H>::ld(wa + i);
-      wvb[j] = Num<H>::ld(wb + i);
+      wva[j] = Num<W>::ld(wa + i);
+      wvb[j] = Num<W>::ld(wb + i);
     }
   }
   float squares = 0.f;
@@ -154,12 +154,15 @@ extern "C" int ts_stream_update_norm(float* x, const void* a, int a_dtype, const
   for (int code : {a_dtype, b_dtype, bias_dtype, h_dtype, w_dtype})
     if (code != 0 && code != 1) return TS_BAD_DTYPE;
   const bool typed = (!a || a_dtype == 0) && (!b || b_dtype == 0) && width <= RS_THREADS * RS_HELD &&
-                     (!bias || bias_dtype == h_dtype || !(h1 || h2)) && (!(h1 || h2) || w_dtype == h_dtype);
+                     (!bias || bias_dtype == h_dtype || !(h1 || h2)) && (!(h1 || h2) || w_dtype == h_dtype || w_dtype == 0);
   if (typed) {
     const int code = (h1 || h2) ? h_dtype : bias_dtype;
+#define RS_TYPED_W(H, W, HELD, NN) \
+  stream_update_norm_held_kernel<H, W, HELD, NN><<<num_rows, RS_THREADS, 0, stream>>>(x, (const float*)a, (const float*)b, \
+      (const H*)bias, mult, (H*)h1, (H*)h2, (const W*)w1, (const W*)w2, eps, rows, width)
+  // (norm weights kept in 32-bit beside outputs in bfloat16: norms whose weights are sums made in 32-bit)
 #define RS_TYPED_N(H, HELD, NN) \
-  stream_update_norm_held_kernel<H, HELD, NN><<<num_rows, RS_THREADS, 0, stream>>>(x, (const float*)a, (const float*)b, \
-      (const H*)bias, mult, (H*)h1, (H*)h2, (const H*)w1, (const H*)w2, eps, rows, width)
+  if (sizeof(H) == 2 && w_dtype == 0 && (h1 || h2)) { RS_TYPED_W(H, float, HELD, NN); } else { RS_TYPED_W(H, H, HELD, NN); }
 #define RS_TYPED(H, HELD) if (h1 || h2) { RS_TYPED_N(H, HELD, true); } else { RS_TYPED_N(H, HELD, false); }
 #define RS_TYPED_H(H) \
   if (width <= RS_THREADS * 4) { RS_TYPED(H, 4); } else if (width <= RS_THREADS * 8) { RS_TYPED(H, 8); } else { RS_TYPED(H, RS_HELD); }
@@ -167,6 +170,7 @@ extern "C" int ts_stream_update_norm(float* x, const void* a, int a_dtype, const
 #undef RS_TYPED_H
 #undef RS_TYPED
 #undef RS_TYPED_N
+#undef RS_TYPED_W
     return ts_check_launch();
   }
   stream_update_norm_kernel<<<num_rows, RS_THREADS, 0, stream>>>(x, a, a_dtype, b, b_dtype, bias, bias_dtype, mult, h1, h2,

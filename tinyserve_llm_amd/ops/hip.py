@@ -2201,7 +2201,7 @@ def latent_mfma_takes(q: torch.Tensor, cache: torch.Tensor, v_cache: torch.Tenso
     return (v_cache is not None and q.dtype == torch.float32 and cache.dtype == torch.bfloat16 and v_cache.dtype == torch.bfloat16
             and cache.shape[1] == 32 and v_cache.stride(1) == 1 and bool(library().ts_latent_mfma_takes(rank, q.shape[2]))
             and all(st % 8 == 0 for st in (cache.stride(0), cache.stride(1), v_cache.stride(0), v_cache.stride(3)))
-            and cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0)
+            and cache.data_ptr() % 16 == 0 and v_cache.data_ptr() % 16 == 0 and q.data_ptr() % 16 == 0)
 
 
 def paged_attention_latent(q: torch.Tensor, cache: torch.Tensor, rank: int, ctx, space: int, scale: float, window: int = 0,
