@@ -720,12 +720,13 @@ def bafarax(args) -> int:
             q32 = torch.randn(T, nh, hd + rot, device="cuda")
             uk = (torch.randn(nh, hd, rank, device="cuda") * 0.05).to(bf)
             uv = (torch.randn(nh, hd, rank, device="cuda") * 0.05).to(bf)
+            uk_t = uk.transpose(1, 2).contiguous()           # (as the part keeps it: a head's dimensions along memory)
             freqs = torch.rand(rot // 2, dtype=torch.float64, device="cuda")
             absorbed = torch.empty(T, nh, row, device="cuda")
             heads = torch.empty(T, nh, hd, dtype=bf, device="cuda")
 
             def before():
-                hip.heads_gemm(q32[:, :, :hd], uk, absorbed[:, :, :rank])
+                hip.heads_gemm(q32[:, :, :hd], uk_t.transpose(1, 2), absorbed[:, :, :rank])
                 hip.rotate_heads(absorbed[:, :, rank:], q32[:, :, hd:], freqs, 1.2, ctx.positions, interleaved=True)
             before()
             attend = lambda: hip.paged_attention_latent(absorbed, cache, rank, ctx, 0, (hd + rot) ** -0.5, window, 0, out_dtype=bf, v_cache=values)

@@ -250,11 +250,12 @@ def test_a_stretch_of_every_head_turns_to_a_place_of_its_own(interleaved):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(1, 3, 24, 40), (5, 3, 20, 34), (23, 2, 16, 16), (70, 8, 64, 256), (130, 4, 128, 512), (300, 2, 33, 65)])
+@pytest.mark.parametrize("sizes", [(1, 3, 24, 40), (5, 3, 20, 34), (23, 2, 16, 16), (70, 8, 64, 256), (130, 4, 128, 512), (300, 2, 33, 65),
+                                   (2, 5, 24, 40), (64, 3, 256, 64), (200, 2, 40, 70)])
 def test_products_per_head_as_stored_and_transposed_with_a_gate(dtype, sizes):
     h = hip()
     T, H, K, N = sizes
-    x = torch.randn(T, H, K + 5)
+    x = torch.randn(T, H, K + (8 if T % 2 == 0 else 5))     # (rows at 16-byte borders, which the matrix cores want, or not)
     w, w64 = rounded(torch.randn(H, K, N) * K ** -0.5, dtype)
     wt, wt64 = rounded(torch.randn(H, N, K) * K ** -0.5, dtype)
     gate = torch.randn(T, H * N + 3) * 2
@@ -265,6 +266,8 @@ def test_products_per_head_as_stored_and_transposed_with_a_gate(dtype, sizes):
     torch.testing.assert_close(out[:, :, :N].cpu().to(F64), torch.einsum("thk,hkn->thn", x.to(F64)[:, :, :K], w64), atol=2e-5, rtol=1e-5)
     assert float(out[:, :, N:].abs().max()) == 0.0
     y = torch.empty(T, H, N, dtype=dtype, device=DEV)
+    # bfloat16 matrices whose k runs along memory, k in 16-byte pieces, aligned rows: the matrix cores
+    assert h.heads_gemm_mfma_takes(xd[:, :, :K], wt.transpose(1, 2), y) == (dtype == torch.bfloat16 and T % 2 == 0 and K % 8 == 0)
     h.heads_gemm(xd[:, :, :K], wt.transpose(1, 2), y, gate=gd[:, :H * N])
     want = torch.einsum("thk,hnk->thn", x.to(F64)[:, :, :K], wt64) * torch.sigmoid(gate.to(F64)[:, :H * N]).view(T, H, N)
     torch.testing.assert_close(y.cpu().to(F64), want, **tol)

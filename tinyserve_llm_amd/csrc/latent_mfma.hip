@@ -320,3 +320,79 @@ extern "C" int ts_paged_attention_latent_mfma(void* out, int out_dtype, const fl
 #undef LM_LAUNCH
   return ts_check_launch();
 }
+
+// ---- products per head on the matrix cores ---------------------------------------------------------------------
+// y[t, h, n] = sum_k x[t, h, k] w[h][n][k] for bfloat16 matrices whose k runs along memory (a matrix stored [k, n]
+// comes as a transposed copy), x 32-bit (rounded to bfloat16 once, as a projection's operand is) or bfloat16, 32-bit
+// sums, times sigmoid(gate) on the way out if there is one. A workgroup makes 64 tokens by 64 columns of one head, a
+// wave 16 tokens: the matrix's rows are the instruction's rows, so that a lane ends with four adjacent columns of
+// one token. Operands come straight from memory in 16-byte pieces; pieces past K are zeros of x against the
+// matrix's last piece.
+#define HM_TOKENS 64
+#define HM_COLS 64
+
+template <typename TX, typename TO>
+__global__ void __launch_bounds__(LM_THREADS)
+heads_gemm_mfma_kernel(TO* __restrict__ y, int64_t y_token, int64_t y_head, const TX* __restrict__ x, int64_t x_token,
+                       int64_t x_head, const bf16_t* __restrict__ w, int64_t w_head, int64_t w_n, int num_tokens, int N, int K,
+                       const float* __restrict__ gate, int64_t gate_token) {
+  const int wave = wave_index(), lane = threadIdx.x & (TS_WAVE - 1);
+  const int r = lane & 15, g = lane >> 4;
+  const int h = blockIdx.y, n0 = blockIdx.z * HM_COLS;
+  const int t = blockIdx.x * HM_TOKENS + 16 * wave + r;
+  const TX* xrow = x + (int64_t)min(t, num_tokens - 1) * x_token + (int64_t)h * x_head;
+  const bf16_t* wh = w + (int64_t)h * w_head;
+  float4_t acc[HM_COLS / 16];
+#pragma unroll
+  for (int nb = 0; nb < HM_COLS / 16; ++nb) acc[nb] = (float4_t){0.f, 0.f, 0.f, 0.f};
+  for (int k0 = 0; k0 < K; k0 += 32) {
+    const int k = k0 + 8 * g, kc = min(k, K - 8);
+    uint4 b;
+    if constexpr (sizeof(TX) == 4) {
+      const float4 lo = *(const float4*)(xrow + kc), hi = *(const float4*)(xrow + kc + 4);
+      b = make_uint4(pack_bf16(lo.x, lo.y), pack_bf16(lo.z, lo.w), pack_bf16(hi.x, hi.y), pack_bf16(hi.z, hi.w));
+    } else {
+      b = *(const uint4*)(xrow + kc);
+    }
+    if (k >= K) b = make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int nb = 0; nb < HM_COLS / 16; ++nb) {
+      const int n = min(n0 + 16 * nb + r, N - 1);
+      acc[nb] = mfma32(*(const uint4*)(wh + (int64_t)n * w_n + kc), b, acc[nb]);
+    }
+  }
+  if (t >= num_tokens) return;
+#pragma unroll
+  for (int nb = 0; nb < HM_COLS / 16; ++nb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int n = n0 + 16 * nb + 4 * g + j;
+      if (n >= N) continue;
+      float v = acc[nb][j];
+      if (gate) v = v / (1.0f + expf(-gate[(int64_t)t * gate_token + (int64_t)h * N + n]));
+      Num<TO>::st(y + (int64_t)t * y_token + (int64_t)h * y_head + n, v);
+    }
+}
+
+// w: bfloat16 [heads][N][K] with K along memory (stride w_n between rows, a multiple of 8; K a multiple of 8);
+// x rows 16-byte aligned.
+extern "C" int ts_heads_gemm_mfma(void* y, int y_dtype, int64_t y_token, int64_t y_head, const void* x, int x_dtype,
+                                  int64_t x_token, int64_t x_head, const void* w, int64_t w_head, int64_t w_n, int num_tokens,
+                                  int heads, int N, int K, const float* gate, int64_t gate_token, hipStream_t stream) {
+  if (num_tokens <= 0) return TS_OK;
+  const int x_size = x_dtype == 0 ? 4 : 2;
+  if (heads <= 0 || heads > 65535 || N <= 0 || K < 8 || K % 8 || w_n % 8 || w_head % 8 || ((uintptr_t)w & 15) ||
+      ((uintptr_t)x & 15) || (x_token * x_size) % 16 || (x_head * x_size) % 16 || (N + HM_COLS - 1) / HM_COLS > 65535)
+    return TS_BAD_SHAPE;
+  dim3 grid((num_tokens + HM_TOKENS - 1) / HM_TOKENS, heads, (N + HM_COLS - 1) / HM_COLS);
+#define HM_LAUNCH(TX, TO) \
+  heads_gemm_mfma_kernel<TX, TO><<<grid, LM_THREADS, 0, stream>>>((TO*)y, y_token, y_head, (const TX*)x, x_token, x_head, \
+      (const bf16_t*)w, w_head, w_n, num_tokens, N, K, gate, gate_token)
+  if (x_dtype == 0 && y_dtype == 0) HM_LAUNCH(float, float);
+  else if (x_dtype == 0 && y_dtype == 1) HM_LAUNCH(float, bf16_t);
+  else if (x_dtype == 1 && y_dtype == 0) HM_LAUNCH(bf16_t, float);
+  else if (x_dtype == 1 && y_dtype == 1) HM_LAUNCH(bf16_t, bf16_t);
+  else return TS_BAD_DTYPE;
+#undef HM_LAUNCH
+  return ts_check_launch();
+}

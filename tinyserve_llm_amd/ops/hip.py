@@ -99,6 +99,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_segment_rmsnorm": [p, i, i64, p, i64, i, p, f, i, p],
         "ts_latent_finish": [p, p, i, p, i64, i, i, i, i, i, p, p, f, p, f, p, p, i, i64, i64, p, i64, i64, i, p],
         "ts_latent_mfma_takes": [i, i],
+        "ts_heads_gemm_mfma": [p, i, i64, i64, p, i, i64, i64, p, i64, i64, i, i, i, i, p, i64, p],
         "ts_paged_attention_latent_mfma": [p, i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i, f, i, i, i, p, p, p],
         "ts_rotate_heads": [p, i, i64, i64, p, i64, i64, i, i, i, p, f, p, i, p],
         "ts_heads_gemm": [p, i, i64, i64, p, i, i64, i64, p, i, i64, i64, i64, i, i, i, i, p, i64, p],
@@ -2173,16 +2174,31 @@ def rotate_heads(dst: torch.Tensor, src: torch.Tensor, freqs: torch.Tensor, ampl
         _ptr(freqs), float(amplitude), _ptr(positions), T, _stream()))
 
 
+def heads_gemm_mfma_takes(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
+    """Whether the matrix-core kernel serves a per-head product: bfloat16 matrices whose k runs along memory, k in whole
+    16-byte pieces, rows of x that start at 16-byte borders."""
+    size = x.element_size()
+    return (w.dtype == torch.bfloat16 and x.dtype in (torch.float32, torch.bfloat16) and out.dtype in (torch.float32, torch.bfloat16)
+            and w.stride(1) == 1 and w.shape[1] >= 8 and w.shape[1] % 8 == 0 and w.stride(2) % 8 == 0 and w.stride(0) % 8 == 0
+            and w.data_ptr() % 16 == 0 and x.data_ptr() % 16 == 0 and (x.stride(0) * size) % 16 == 0 and (x.stride(1) * size) % 16 == 0)
+
+
 def heads_gemm(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, gate: torch.Tensor | None = None) -> torch.Tensor:
     """out[t, h, :] = x[t, h, :] · w[h] with w [heads, k, n] (any strides: a transposed view multiplies by the
-    transpose), 32-bit multiply-adds in ascending k. x [tokens, heads, k] and out [tokens, heads, n] are views whose
-    last dimension is contiguous. `gate` (float32 [tokens, heads * n], rows may lie apart): out is multiplied by
-    sigmoid(gate) on its way out."""
+    transpose). x [tokens, heads, k] and out [tokens, heads, n] are views whose last dimension is contiguous. `gate`
+    (float32 [tokens, heads * n], rows may lie apart): out is multiplied by sigmoid(gate) on its way out. bfloat16
+    matrices whose k runs along memory go to the matrix cores (x rounded to bfloat16 once, 32-bit sums); everything
+    else is 32-bit multiply-adds in ascending k."""
     _gpu(x, w, out, gate)
     T, H, K = x.shape
     N = w.shape[2]
     _need(w.dim() == 3 and w.shape[0] == H and w.shape[1] == K and out.shape == (T, H, N), "x [tokens, heads, k], w [heads, k, n], out [tokens, heads, n]")
     _need(x.stride(2) == 1 and out.stride(2) == 1, "rows of x and out must be contiguous")
+    if heads_gemm_mfma_takes(x, w, out):
+        _run("heads_gemm_mfma", library().ts_heads_gemm_mfma(
+            _ptr(out), _code(out.dtype), out.stride(0), out.stride(1), _ptr(x), _code(x.dtype), x.stride(0), x.stride(1), _ptr(w),
+            w.stride(0), w.stride(2), T, H, N, K, _ptr(gate), _check_gate(gate, T, H * N), _stream()))
+        return out
     _run("heads_gemm", library().ts_heads_gemm(
         _ptr(out), _code(out.dtype), out.stride(0), out.stride(1), _ptr(x), _code(x.dtype), x.stride(0), x.stride(1), _ptr(w),
         _code(w.dtype), *w.stride(), T, H, N, K, _ptr(gate), _check_gate(gate, T, H * N), _stream()))

@@ -46,6 +46,12 @@ class LatentAttention(Mixer):
         self.uv: torch.Tensor | None = None
         self.o: torch.Tensor | None = None
         self.down_packed = self.uq_packed = self.o_packed = None
+        self.uk_t: torch.Tensor | None = None      # W_uk per head with the head's dimensions along memory, for the matrix cores
+
+    def bind(self, params) -> None:
+        super().bind(params)
+        if self.uk is not None and self.uk.dtype == torch.bfloat16 and self.uk.is_cuda:
+            self.uk_t = self.uk.view(self.num_heads, self.head_dim, self.kv_rank).transpose(1, 2).contiguous()
 
     @property
     def out_size(self) -> int:
@@ -91,7 +97,7 @@ class LatentAttention(Mixer):
         q = linear(cq, self.uq, out_dtype=torch.float32, packed=self.uq_packed).view(T, H, D + R)
         # the keys' up-projection on the query's side: W_uk,h^T q_h beside the turned part, in the cached row's order
         absorbed = torch.empty((T, H, C + R), dtype=torch.float32, device=x.device)
-        hip.heads_gemm(q[:, :, :D], self.uk.view(H, D, C), absorbed[:, :, :C])
+        hip.heads_gemm(q[:, :, :D], self.uk.view(H, D, C) if self.uk_t is None else self.uk_t.transpose(1, 2), absorbed[:, :, :C])
         if R:
             hip.rotate_heads(absorbed[:, :, C:], q[:, :, D:], freqs, amplitude, ctx.positions, interleaved=True)
         mixed = hip.paged_attention_latent(absorbed, mem.k_cache, C, ctx, mem.space, self.scale, self.window, self.chunk, out_dtype=x.dtype,
