@@ -345,6 +345,7 @@ heads_gemm_mfma_kernel(TO* __restrict__ y, int64_t y_token, int64_t y_head, cons
   float4_t acc[HM_COLS / 16];
 #pragma unroll
   for (int nb = 0; nb < HM_COLS / 16; ++nb) acc[nb] = (float4_t){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
   for (int k0 = 0; k0 < K; k0 += 32) {
     const int k = k0 + 8 * g, kc = min(k, K - 8);
     uint4 b;
