@@ -152,7 +152,7 @@ def decides(want_row, value_row) -> bool:
 @pytest.mark.parametrize("form", sorted(FORMS))
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("chunk, sizes", [(1, (4, 2, 32, 40)), (7, (4, 2, 32, 40)), (16, (4, 2, 32, 40)), (24, (4, 2, 32, 40)),
-                                          (64, (8, 1, 64, 64)), (100, (4, 2, 32, 40)), (33, (8, 2, 64, 64)), (65, (4, 4, 64, 64)),
+                                          (64, (8, 2, 64, 64)), (100, (4, 2, 32, 40)), (33, (8, 2, 64, 64)), (65, (4, 4, 64, 64)),
                                           (130, (4, 1, 64, 64)), (96, (2, 2, 128, 128)), (257, (6, 2, 32, 32)), (3, (3, 1, 20, 12))])
 def test_chunk_edges(dtype, chunk, sizes, form):
     """The key that stands out is the first of the query's chunk for some queries (the farthest key they see) and the last
@@ -179,7 +179,7 @@ def test_chunk_edges(dtype, chunk, sizes, form):
 
 @pytest.mark.parametrize("form", sorted(FORMS))
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(4, 2, 32, 48), (2, 2, 16, 16), (6, 1, 24, 8), (8, 1, 64, 64), (4, 4, 128, 128)])
+@pytest.mark.parametrize("sizes", [(4, 2, 32, 48), (2, 2, 16, 16), (6, 1, 24, 8), (8, 4, 64, 64), (4, 4, 128, 128)])
 def test_far_keys_and_page_borders_without_chunks_and_inside_a_long_chunk(dtype, sizes, form):
     H, G, D, V = sizes
     page, length = 16, 700
@@ -315,8 +315,8 @@ def latent_case(dtype, H, rank, rot, page, length, queries, stand_out, scale, wi
 @pytest.mark.parametrize("form", sorted(FORMS))
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("page", [16, 32])
-@pytest.mark.parametrize("window, sizes", [(1, (3, 40, 8)), (7, (3, 34, 6)), (16, (2, 16, 16)), (50, (3, 48, 8)), (64, (4, 128, 16)),
-                                           (70, (5, 16, 16)), (96, (4, 128, 16)), (130, (8, 256, 32)), (257, (2, 512, 64)), (65, (4, 64, 0)),
+@pytest.mark.parametrize("window, sizes", [(1, (3, 40, 8)), (7, (3, 34, 6)), (16, (2, 16, 16)), (50, (3, 48, 8)), (64, (4, 96, 16)),
+                                           (70, (5, 16, 16)), (96, (6, 128, 32)), (130, (8, 256, 32)), (257, (2, 512, 64)), (65, (4, 64, 0)),
                                            (33, (24, 32, 8)), (100, (32, 256, 64)), (31, (16, 80, 24)), (200, (40, 64, 8))])
 def test_latent_attention_window_edges(dtype, window, sizes, form, page):
     """Pages of 16 keys go to the kernel that is 32-bit throughout, as float32 always does; pages of 32 in bfloat16 go to
@@ -372,7 +372,7 @@ def mlstm_weights(H, D, V, cap):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("sizes", [(3, 20, 28, 8.0), (1, 16, 16, 15.0), (2, 18, 270, 5.0), (4, 64, 128, 12.0), (2, 32, 48, 12.0),
+@pytest.mark.parametrize("sizes", [(3, 20, 28, 8.0), (1, 16, 16, 15.0), (2, 18, 270, 5.0), (4, 64, 128, 12.0), (2, 32, 40, 10.0),
                                    (1, 1, 1, 2.0), (2, 128, 64, 6.0), (1, 300, 20, 4.0)])
 @pytest.mark.parametrize("portions", [[1, 2, 13, 1, 5, 31, 3], [1, 2, 13, 1, 5, 64, 3], [200, 1, 32]])
 def test_matrix_memory_over_steps_slots_and_gates_at_their_caps(dtype, sizes, portions):
