@@ -762,8 +762,7 @@ def bafarax(args) -> int:
                 return out
 
             def baf_finish():
-                hip.segment_rmsnorm(plain32, 0, nh * hd, qw, 1e-6, out=plain32[:, :nh * hd])
-                hip.segment_rmsnorm(plain32, nh * hd, nkv * hd, kw, 1e-6, out=plain32[:, nh * hd:(nh + nkv) * hd])
+                hip.segment_rmsnorm_pair(plain32, (0, nh * hd, qw), (nh * hd, nkv * hd, kw), 1e-6)
                 return hip.qkv_finish(plain32, rfreqs, ctx.positions, slots, k, v, nh, nkv, hd, hd, bf, interleaved=False)
             down = torch.randn(T, q_rank + row + nh * hd, device="cuda")
             lqw, lcw = torch.ones(q_rank, device="cuda"), torch.ones(rank, device="cuda")

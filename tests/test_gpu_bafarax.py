@@ -68,6 +68,9 @@ def test_norm_over_a_whole_projection_in_place(sizes):
     torch.testing.assert_close(d[:, :q].cpu().to(F64), plain.unit_rms(r[:, :q], 1e-5) * wq.to(F64), atol=5e-6, rtol=1e-5)
     torch.testing.assert_close(d[:, q:q + k].cpu().to(F64), plain.unit_rms(r[:, q:q + k], 1e-5) * wk.to(F64), atol=5e-6, rtol=1e-5)
     assert torch.equal(d[:, q + k:].cpu(), rows[:, q + k:]), "the values are left as they are"
+    both = rows.to(DEV)
+    h.segment_rmsnorm_pair(both, (0, q, wq.to(DEV)), (q, k, wk.to(DEV)), 1e-5)              # the two in one launch
+    assert torch.equal(both, d)
     out = h.segment_rmsnorm(rows.to(DEV), q, k, None, 0.0, out_dtype=torch.bfloat16)
     torch.testing.assert_close(out.cpu().to(F64), plain.unit_rms(r[:, q:q + k], 0.0), atol=2e-2, rtol=1e-2)
 

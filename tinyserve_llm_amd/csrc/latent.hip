@@ -58,6 +58,29 @@ extern "C" int ts_segment_rmsnorm(void* out, int out_dtype, int64_t out_stride, 
   return ts_check_launch();
 }
 
+// Two stretches of every row in one launch, in place (the norms over a token's whole q and whole k projection):
+// workgroup (row, 0) takes the first, (row, 1) the second.
+__global__ void __launch_bounds__(LT_THREADS)
+segment_rmsnorm_pair_kernel(float* __restrict__ x, int64_t x_stride, int off0, int size0, const float* __restrict__ w0, int off1,
+                            int size1, const float* __restrict__ w1, float eps) {
+  __shared__ float red[LT_WAVES];
+  const int off = blockIdx.y ? off1 : off0, size = blockIdx.y ? size1 : size0;
+  const float* weight = blockIdx.y ? w1 : w0;
+  float* row = x + (int64_t)blockIdx.x * x_stride + off;
+  float squares = 0.f;
+  for (int d = threadIdx.x; d < size; d += LT_THREADS) squares = fmaf(row[d], row[d], squares);
+  const float inv = 1.0f / sqrtf(lt_block_sum(squares, red) / (float)size + eps);
+  for (int d = threadIdx.x; d < size; d += LT_THREADS) row[d] = row[d] * inv * weight[d];
+}
+
+extern "C" int ts_segment_rmsnorm_pair(float* x, int64_t x_stride, int off0, int size0, const float* w0, int off1, int size1,
+                                       const float* w1, float eps, int num_rows, hipStream_t stream) {
+  if (num_rows <= 0) return TS_OK;
+  if (size0 <= 0 || size1 <= 0 || off0 < 0 || off1 < off0 + size0 || off1 + size1 > x_stride || !w0 || !w1) return TS_BAD_SHAPE;
+  segment_rmsnorm_pair_kernel<<<dim3(num_rows, 2), LT_THREADS, 0, stream>>>(x, x_stride, off0, size0, w0, off1, size1, w1, eps);
+  return ts_check_launch();
+}
+
 // The angle position * f in 64-bit, brought to [-pi, pi] before the 32-bit sine and cosine.
 static __device__ __forceinline__ void lt_angle(int pos, double f, float amplitude, float* cs, float* sn) {
   const double angle = (double)pos * f;

@@ -97,6 +97,7 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_moe_group": [p, p, p, i, i, i, i, p],
         "ts_moe_gemm": [p, i, p, i, p, p, p, i, i, i, i, i, i, f, f, f, i, p],
         "ts_segment_rmsnorm": [p, i, i64, p, i64, i, p, f, i, p],
+        "ts_segment_rmsnorm_pair": [p, i64, i, i, p, i, i, p, f, i, p],
         "ts_latent_finish": [p, p, i, p, i64, i, i, i, i, i, p, p, f, p, f, p, p, i, i64, i64, p, i64, i64, i, p],
         "ts_latent_mfma_takes": [i, i],
         "ts_heads_gemm_mfma": [p, i, i64, i64, p, i, i64, i64, p, i64, i64, i, i, i, i, p, i64, p],
@@ -2100,6 +2101,19 @@ def segment_rmsnorm(x: torch.Tensor, offset: int, size: int, weight: torch.Tenso
         _ptr(out), _code(out.dtype), out.stride(0) if x.shape[0] > 1 else size, x.data_ptr() + 4 * offset,
         x.stride(0) if x.shape[0] > 1 else x.shape[1], size, _ptr(weight), float(eps), x.shape[0], _stream()))
     return out
+
+
+def segment_rmsnorm_pair(x: torch.Tensor, first: tuple[int, int, torch.Tensor], second: tuple[int, int, torch.Tensor], eps: float) -> None:
+    """Two stretches (offset, size, weight float32 [size]) of every row of x (contiguous float32 [rows, width]), the second
+    behind the first, each divided by its own root mean square and multiplied by its weight, in place, in one launch."""
+    _gpu(x, first[2], second[2])
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous(), "contiguous rows of float32")
+    for off, size, w in (first, second):
+        _need(w.dtype == torch.float32 and w.shape == (size,) and w.is_contiguous(), "a weight must be float32 [size]")
+    _need(0 <= first[0] and first[1] > 0 and second[1] > 0 and first[0] + first[1] <= second[0] and second[0] + second[1] <= x.shape[1],
+          "two stretches inside a row, one behind the other")
+    _run("segment_rmsnorm_pair", library().ts_segment_rmsnorm_pair(_ptr(x), x.shape[1], first[0], first[1], _ptr(first[2]), second[0], second[1],
+                                                                   _ptr(second[2]), float(eps), x.shape[0], _stream()))
 
 
 def _check_step_vectors(T: int, **vectors: torch.Tensor | None) -> None:

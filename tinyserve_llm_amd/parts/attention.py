@@ -207,9 +207,7 @@ class GeneralAttention(Mixer):
         k_store, v_store = (mem.k_cache, mem.v_cache) if mem.store else (None, None)
         qkv = linear(x, self.qkv, out_dtype=torch.float32, packed=self.qkv_packed)
         if self.projection_norm_eps is not None:         # in place, each over its whole stretch of the row
-            hip.segment_rmsnorm(qkv, 0, self.q_size, self.q_norm, self.projection_norm_eps, out=qkv[:, :self.q_size])
-            hip.segment_rmsnorm(qkv, self.q_size, self.k_size, self.k_norm, self.projection_norm_eps,
-                                out=qkv[:, self.q_size:self.q_size + self.k_size])
+            hip.segment_rmsnorm_pair(qkv, (0, self.q_size, self.q_norm), (self.q_size, self.k_size, self.k_norm), self.projection_norm_eps)
         q = hip.qkv_finish(qkv, enc.frequencies() if enc is not None else None, ctx.positions, slots, k_store, v_store,
                            self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, x.dtype,
                            interleaved=getattr(enc, "interleaved", True), qk_norm_eps=self.qk_norm_eps,
