@@ -431,3 +431,59 @@ extern "C" int ts_paged_attention_general(void* out, const void* q, const void* 
     return TS_BAD_DTYPE;
   return ts_check_launch();
 }
+
+// ---- what some designs do to the projected rows before q and k turn ----
+// In place on the 32-bit rows q | k | v of a step, one wave per (token, head):
+//   * each q head and each k head divided by its root mean square (eps inside the root) and multiplied by a weight
+//     of the head's size that all heads share (q_weight / k_weight; absent: that kind of head is left alone);
+//   * each value head turned by the token's position over all its dimensions (v_freqs [vd / 2], 64-bit; pair m is
+//     dimensions (m, m + vd/2), or (2m, 2m + 1) if `v_interleaved`), so that the cache holds rotated values.
+__global__ void __launch_bounds__(AG_WAVES * TS_WAVE)
+qkv_prepare_kernel(float* __restrict__ qkv, const int32_t* __restrict__ positions, int nh, int nkv, int hd, int vd_size,
+                   const float* __restrict__ q_weight, const float* __restrict__ k_weight, float eps,
+                   const double* __restrict__ v_freqs, int v_interleaved, int64_t items) {
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
+  const int64_t item = (int64_t)blockIdx.x * AG_WAVES + wave;
+  if (item >= items) return;
+  const int heads = nh + 2 * nkv;
+  const int64_t t = item / heads;
+  const int h = (int)(item - t * heads);
+  const int64_t row = (int64_t)(nh + nkv) * hd + (int64_t)nkv * vd_size;
+  if (h < nh + nkv) {
+    const float* weight = h < nh ? q_weight : k_weight;
+    if (!weight) return;
+    float* head = qkv + t * row + (int64_t)h * hd;
+    float squares = 0.f;
+    for (int d = lane; d < hd; d += TS_WAVE) squares = fmaf(head[d], head[d], squares);
+    const float inv = 1.0f / sqrtf(wave_sum(squares) / (float)hd + eps);
+    for (int d = lane; d < hd; d += TS_WAVE) head[d] = head[d] * inv * weight[d];
+    return;
+  }
+  if (!v_freqs) return;
+  float* head = qkv + t * row + (int64_t)(nh + nkv) * hd + (int64_t)(h - nh - nkv) * vd_size;
+  const int half = vd_size / 2;
+  const int pos = positions[t];
+  for (int pair = lane; pair < half; pair += TS_WAVE) {
+    const double angle = (double)pos * v_freqs[pair];
+    const double turns = rint(angle * 0.15915494309189535);
+    float sn, cs;
+    sincosf((float)fma(-turns, 6.283185307179586, angle), &sn, &cs);
+    const int a = v_interleaved ? 2 * pair : pair, b = v_interleaved ? 2 * pair + 1 : pair + half;
+    const float u = head[a], v = head[b];
+    head[a] = u * cs - v * sn;
+    head[b] = v * cs + u * sn;
+  }
+}
+
+extern "C" int ts_qkv_prepare(float* qkv, const int32_t* positions, int num_tokens, int nh, int nkv, int hd, int vd_size,
+                              const float* q_weight, const float* k_weight, float eps, const double* v_freqs,
+                              int v_interleaved, hipStream_t stream) {
+  if (num_tokens <= 0 || (!q_weight && !k_weight && !v_freqs)) return TS_OK;
+  if (nh <= 0 || nkv <= 0 || hd <= 0 || vd_size <= 0 || (v_freqs && vd_size % 2)) return TS_BAD_SHAPE;
+  const int64_t items = (int64_t)num_tokens * (nh + 2 * nkv);
+  const int64_t blocks = (items + AG_WAVES - 1) / AG_WAVES;
+  if (blocks > 0x7fffffff) return TS_BAD_SHAPE;
+  qkv_prepare_kernel<<<(unsigned)blocks, AG_WAVES * TS_WAVE, 0, stream>>>(qkv, positions, nh, nkv, hd, vd_size, q_weight, k_weight,
+                                                                         eps, v_freqs, v_interleaved, items);
+  return ts_check_launch();
+}

@@ -169,7 +169,7 @@ extern "C" int ts_embedding_dyt_stream(float* out, const void* table, int dtype,
 // limit <= 0: no cap. Rows may be picked through `row_stride` (a row of the operand may be wider than 2 ff).
 __global__ void __launch_bounds__(DT_THREADS)
 capped_glu_kernel(void* __restrict__ out, int out_code, const void* __restrict__ gate_up, int in_code, int64_t row_stride,
-                  int ff, float limit, float slope, float up_shift, int64_t total) {
+                  int ff, float limit, float slope, float up_shift, int64_t total, int relu) {
   const int64_t at = (int64_t)blockIdx.x * DT_THREADS + threadIdx.x;
   if (at >= total) return;
   const int64_t t = at / ff;
@@ -180,12 +180,13 @@ capped_glu_kernel(void* __restrict__ out, int out_code, const void* __restrict__
     g = fminf(g, limit);
     u = fminf(fmaxf(u, -limit), limit);
   }
-  const float y = g / (1.0f + expf(-slope * g)) * (u + up_shift);
+  // (`relu`: the gate passes where it is positive, max(g, 0) (u + up_shift), instead of through a sigmoid)
+  const float y = (relu ? fmaxf(g, 0.f) : g / (1.0f + expf(-slope * g))) * (u + up_shift);
   dt_store(out, out_code, at, y);
 }
 
 extern "C" int ts_capped_glu(void* out, int out_dtype, const void* gate_up, int in_dtype, int64_t row_stride, int n, int ff,
-                             float limit, float slope, float up_shift, hipStream_t stream) {
+                             float limit, float slope, float up_shift, int relu, hipStream_t stream) {
   if (n <= 0) return TS_OK;
   if (ff <= 0 || row_stride < 2 * (int64_t)ff) return TS_BAD_SHAPE;
   if ((out_dtype | in_dtype) & ~1) return TS_BAD_DTYPE;
@@ -193,6 +194,6 @@ extern "C" int ts_capped_glu(void* out, int out_dtype, const void* gate_up, int 
   const int64_t blocks = (total + DT_THREADS - 1) / DT_THREADS;
   if (blocks > 0x7fffffff) return TS_BAD_SHAPE;
   capped_glu_kernel<<<(unsigned)blocks, DT_THREADS, 0, stream>>>(out, out_dtype, gate_up, in_dtype, row_stride, ff, limit, slope,
-                                                                 up_shift, total);
+                                                                 up_shift, total, relu);
   return ts_check_launch();
 }

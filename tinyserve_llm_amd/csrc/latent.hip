@@ -150,12 +150,14 @@ extern "C" int ts_latent_finish(void* cq_out, void* cache, int out_dtype, const 
   return ts_check_launch();
 }
 
-// One thread per (token, head, pair).
-template <typename TO>
+// One thread per (token, head, pair). `back`: by minus the angle. `gate` (32-bit, a number per token and head,
+// `gate_token` apart from token to token): the turned pair is multiplied by sigmoid(gate[t, h]).
+template <typename TI, typename TO>
 __global__ void __launch_bounds__(LT_THREADS)
-rotate_heads_kernel(TO* __restrict__ dst, int64_t dst_token, int64_t dst_head, const float* __restrict__ src, int64_t src_token,
+rotate_heads_kernel(TO* __restrict__ dst, int64_t dst_token, int64_t dst_head, const TI* __restrict__ src, int64_t src_token,
                     int64_t src_head, int heads, int rot, int interleaved, const double* __restrict__ freqs, float amplitude,
-                    const int32_t* __restrict__ positions, int64_t items) {
+                    const int32_t* __restrict__ positions, int64_t items, int back, const float* __restrict__ gate,
+                    int64_t gate_token) {
   const int64_t item = (int64_t)blockIdx.x * LT_THREADS + threadIdx.x;
   if (item >= items) return;
   const int half = rot / 2;
@@ -164,27 +166,31 @@ rotate_heads_kernel(TO* __restrict__ dst, int64_t dst_token, int64_t dst_head, c
   const int64_t t = item / ((int64_t)half * heads);
   float cs, sn;
   lt_angle(positions[t], freqs[pair], amplitude, &cs, &sn);
+  if (back) sn = -sn;
+  const float g = gate ? 1.0f / (1.0f + expf(-gate[t * gate_token + h])) : 1.0f;
   const int a = interleaved ? 2 * pair : pair, b = interleaved ? 2 * pair + 1 : pair + half;
-  const float* s = src + t * src_token + h * src_head;
+  const TI* s = src + t * src_token + h * src_head;
   TO* d = dst + t * dst_token + h * dst_head;
-  const float u = s[a], v = s[b];
-  Num<TO>::st(d + a, u * cs - v * sn);
-  Num<TO>::st(d + b, v * cs + u * sn);
+  const float u = Num<TI>::ld(s + a), v = Num<TI>::ld(s + b);
+  Num<TO>::st(d + a, (u * cs - v * sn) * g);
+  Num<TO>::st(d + b, (v * cs + u * sn) * g);
 }
 
-extern "C" int ts_rotate_heads(void* dst, int out_dtype, int64_t dst_token, int64_t dst_head, const float* src,
+extern "C" int ts_rotate_heads(void* dst, int out_dtype, int64_t dst_token, int64_t dst_head, const void* src, int in_dtype,
                                int64_t src_token, int64_t src_head, int heads, int rot, int interleaved, const double* freqs,
-                               float amplitude, const int32_t* positions, int num_tokens, hipStream_t stream) {
+                               float amplitude, const int32_t* positions, int num_tokens, int back, const float* gate,
+                               int64_t gate_token, hipStream_t stream) {
   if (num_tokens <= 0 || rot == 0) return TS_OK;
   if (heads <= 0 || rot < 0 || rot % 2 || !freqs) return TS_BAD_SHAPE;
   const int64_t items = (int64_t)num_tokens * heads * (rot / 2);
   const int64_t blocks = (items + LT_THREADS - 1) / LT_THREADS;
   if (blocks > 0x7fffffff) return TS_BAD_SHAPE;
-#define LT_ROTATE(TO) \
-  rotate_heads_kernel<TO><<<(unsigned)blocks, LT_THREADS, 0, stream>>>((TO*)dst, dst_token, dst_head, src, src_token, src_head, heads, \
-      rot, interleaved, freqs, amplitude, positions, items)
-  if (out_dtype == 0) LT_ROTATE(float);
-  else if (out_dtype == 1) LT_ROTATE(bf16_t);
+#define LT_ROTATE(TI, TO) \
+  rotate_heads_kernel<TI, TO><<<(unsigned)blocks, LT_THREADS, 0, stream>>>((TO*)dst, dst_token, dst_head, (const TI*)src, src_token, \
+      src_head, heads, rot, interleaved, freqs, amplitude, positions, items, back, gate, gate_token)
+  if (in_dtype == 0 && out_dtype == 0) LT_ROTATE(float, float);
+  else if (in_dtype == 0 && out_dtype == 1) LT_ROTATE(float, bf16_t);
+  else if (in_dtype == 1 && out_dtype == 1) LT_ROTATE(bf16_t, bf16_t);
   else return TS_BAD_DTYPE;
 #undef LT_ROTATE
   return ts_check_launch();

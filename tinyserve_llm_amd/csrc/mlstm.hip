@@ -153,11 +153,13 @@ extern "C" int ts_mlstm_scan(float* out, const float* proj, int64_t stride, cons
   return ts_check_launch();
 }
 
-// One wave per (token, head).
+// One wave per (token, head). `weight_head`: elements between two heads' weights (0: one weight of a head's size that all
+// heads share; null weight: none). `silu_gate`: the gate is g sigmoid(g) instead of sigmoid(g).
 template <typename TO>
 __global__ void __launch_bounds__(ML_THREADS)
 mlstm_finish_kernel(TO* __restrict__ out, const float* __restrict__ o, const float* __restrict__ weight,
-                    const float* __restrict__ gate, int64_t gate_stride, int heads, int vdim, float eps, int64_t items) {
+                    const float* __restrict__ gate, int64_t gate_stride, int heads, int vdim, float eps, int64_t items,
+                    int weight_head, int silu_gate) {
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
   const int64_t item = (int64_t)blockIdx.x * ML_WAVES + wave;
   if (item >= items) return;
@@ -169,21 +171,24 @@ mlstm_finish_kernel(TO* __restrict__ out, const float* __restrict__ o, const flo
   const float inv = 1.0f / sqrtf(wave_sum(squares) / (float)vdim + eps);
   for (int d = lane; d < vdim; d += TS_WAVE) {
     const float g = gate[t * gate_stride + h * vdim + d];
-    Num<TO>::st(out + item * vdim + d, row[d] * inv * weight[h * vdim + d] / (1.0f + expf(-g)));
+    const float w = weight ? weight[h * weight_head + d] : 1.0f;
+    const float s = 1.0f / (1.0f + expf(-g));
+    Num<TO>::st(out + item * vdim + d, row[d] * inv * w * (silu_gate ? g * s : s));
   }
 }
 
 extern "C" int ts_mlstm_finish(void* out, int out_dtype, const float* o, const float* weight, const float* gate,
-                               int64_t gate_stride, int num_tokens, int heads, int vdim, float eps, hipStream_t stream) {
+                               int64_t gate_stride, int num_tokens, int heads, int vdim, float eps, int weight_head,
+                               int silu_gate, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
-  if (heads <= 0 || vdim <= 0) return TS_BAD_SHAPE;
+  if (heads <= 0 || vdim <= 0 || (weight_head != 0 && weight_head != vdim)) return TS_BAD_SHAPE;
   const int64_t items = (int64_t)num_tokens * heads;
   const int64_t blocks = (items + ML_WAVES - 1) / ML_WAVES;
   if (blocks > 0x7fffffff) return TS_BAD_SHAPE;
   if (out_dtype == 0)
-    mlstm_finish_kernel<float><<<(unsigned)blocks, ML_THREADS, 0, stream>>>((float*)out, o, weight, gate, gate_stride, heads, vdim, eps, items);
+    mlstm_finish_kernel<float><<<(unsigned)blocks, ML_THREADS, 0, stream>>>((float*)out, o, weight, gate, gate_stride, heads, vdim, eps, items, weight_head, silu_gate);
   else if (out_dtype == 1)
-    mlstm_finish_kernel<bf16_t><<<(unsigned)blocks, ML_THREADS, 0, stream>>>((bf16_t*)out, o, weight, gate, gate_stride, heads, vdim, eps, items);
+    mlstm_finish_kernel<bf16_t><<<(unsigned)blocks, ML_THREADS, 0, stream>>>((bf16_t*)out, o, weight, gate, gate_stride, heads, vdim, eps, items, weight_head, silu_gate);
   else return TS_BAD_DTYPE;
   return ts_check_launch();
 }

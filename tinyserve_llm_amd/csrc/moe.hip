@@ -2,7 +2,9 @@
 //   * `ts_moe_route`: router logits z = W_r h in 32-bit (h as it is stored), scores s = sigmoid(z); the `top`
 //     experts with the largest s + correction are chosen (ties: the lower index); their weights are their s,
 //     divided by the chosen ones' sum (+ 1e-20) if `normalize`, times `scale`. With `softmax_chosen` the logits
-//     themselves are the scores, and the weights are the softmax over the chosen experts' logits alone.
+//     themselves are the scores, and the weights are the softmax over the chosen experts' logits alone. With
+//     `scoring` 2 the scores are the softmax over all the router's outputs. The router may have `extras` more rows
+//     than experts: their logits' sigmoids are left beside the choice (a gate on a shared expert, say).
 //   * `ts_moe_group`: the step's (token, choice) pairs grouped by expert, and the groups cut into tiles of rows
 //     that one workgroup of the product takes: [expert, first index, rows] per tile, rows 0 for the tiles of the
 //     launch that the step does not fill (the launch is sized for the worst case, so nothing comes back to the host).
@@ -12,7 +14,8 @@
 //     Without `glu`, `act` 1 squares the sums' positive parts on their way out (experts of the form W_down relu(W_up h)^2).
 //     Every row's sums run over k in ascending order whatever the tile it lands in.
 //   * `ts_moe_combine`: out[token] = sum over its choices, in order, of weight * the pair's row (+ a shared
-//     expert's row).
+//     expert's row, times a gate per token if there is one). A choice at or beyond `real` is an identity expert: it
+//     has no matrices, `ts_moe_group` leaves its pairs out of every tile, and its row is the token's input itself.
 // float32 runs 32-bit multiply-adds; bfloat16 operands go through the matrix cores with 32-bit sums.
 #include "common.h"
 
@@ -28,15 +31,17 @@ template <typename TX>
 __global__ void __launch_bounds__(MOE_ROUTE_THREADS)
 moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const TX* __restrict__ x,
                  const float* __restrict__ router, const float* __restrict__ correction, int num_tokens, int K, int E, int top,
-                 float scale, int normalize, int softmax_chosen) {
+                 float scale, int normalize, int scoring, int extras, float* __restrict__ extra_out) {
+  const bool softmax_chosen = scoring == 1;
+  const int rows = E + extras;                            // rows of the router: the experts, then the extras
   extern __shared__ float lds[];
-  float* s_s = lds;                                       // [MOE_ROUTE_TOKENS][E] logits, then scores
-  float* c_s = lds + MOE_ROUTE_TOKENS * E;                // [MOE_ROUTE_TOKENS][E] choice scores
-  float* x_s = c_s + MOE_ROUTE_TOKENS * E;                // [MOE_ROUTE_TOKENS][MOE_ROUTE_CHUNK] the tokens' rows, 32-bit
+  float* s_s = lds;                                       // [MOE_ROUTE_TOKENS][rows] logits, then scores
+  float* c_s = lds + MOE_ROUTE_TOKENS * rows;             // [MOE_ROUTE_TOKENS][rows] choice scores
+  float* x_s = c_s + MOE_ROUTE_TOKENS * rows;                // [MOE_ROUTE_TOKENS][MOE_ROUTE_CHUNK] the tokens' rows, 32-bit
   const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
   const int t0 = blockIdx.x * MOE_ROUTE_TOKENS;
   const int nt = min(MOE_ROUTE_TOKENS, num_tokens - t0);
-  for (int i = threadIdx.x; i < MOE_ROUTE_TOKENS * E; i += MOE_ROUTE_THREADS) s_s[i] = 0.f;
+  for (int i = threadIdx.x; i < MOE_ROUTE_TOKENS * rows; i += MOE_ROUTE_THREADS) s_s[i] = 0.f;
   const bool by4 = K % 4 == 0 && ((uintptr_t)router & 15) == 0;     // (rows of the router in 16-byte pieces)
   // a stretch of the rows into LDS, then every wave takes experts in turn: a lane reads the router's row side by
   // side with its neighbours, all of a stretch's pieces asked for before the first is used
@@ -49,7 +54,7 @@ moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const
       x_s[r * MOE_ROUTE_CHUNK + k] = r < nt ? Num<TX>::ld(x + (int64_t)(t0 + r) * K + k0 + k) : 0.f;
     }
     __syncthreads();
-    for (int e = wave; e < E; e += MOE_ROUTE_THREADS / TS_WAVE) {
+    for (int e = wave; e < rows; e += MOE_ROUTE_THREADS / TS_WAVE) {
       float acc[MOE_ROUTE_TOKENS];
 #pragma unroll
       for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) acc[r] = 0.f;
@@ -83,19 +88,38 @@ moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const
 #pragma unroll
       for (int r = 0; r < MOE_ROUTE_TOKENS; ++r) {
         const float z = wave_sum(acc[r]);
-        if (lane == 0) s_s[r * E + e] += z;                // (an expert is one wave's: no other adds to it)
+        if (lane == 0) s_s[r * rows + e] += z;                // (an expert is one wave's: no other adds to it)
       }
     }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < MOE_ROUTE_TOKENS * E; i += MOE_ROUTE_THREADS) {
-    const float sc = softmax_chosen ? s_s[i] : 1.0f / (1.0f + expf(-s_s[i]));
+  for (int i = threadIdx.x; i < MOE_ROUTE_TOKENS * rows; i += MOE_ROUTE_THREADS) {
+    const int e = i % rows;
+    const float sc = (softmax_chosen || (scoring == 2 && e < E)) ? s_s[i] : 1.0f / (1.0f + expf(-s_s[i]));
     s_s[i] = sc;
-    c_s[i] = sc + (correction ? correction[i % E] : 0.f);
+    c_s[i] = sc + ((correction && e < E) ? correction[e] : 0.f);
   }
   __syncthreads();
   if (wave >= nt) return;                                 // a wave per token from here on
   const int r = wave, t = t0 + wave;
+  s_s += r * rows;
+  c_s += r * rows;
+  if (extras && lane < extras) extra_out[(int64_t)t * extras + lane] = s_s[E + lane];
+  if (scoring == 2) {                                     // the softmax over all the experts' logits
+    float top_logit = -INFINITY;
+    for (int e = lane; e < E; e += TS_WAVE) top_logit = fmaxf(top_logit, s_s[e]);
+    top_logit = wave_max(top_logit);
+    float total = 0.f;
+    for (int e = lane; e < E; e += TS_WAVE) total += expf(s_s[e] - top_logit);
+    total = wave_sum(total);
+    wave_sync();
+    for (int e = lane; e < E; e += TS_WAVE) {
+      const float sc = expf(s_s[e] - top_logit) / total;
+      s_s[e] = sc;
+      c_s[e] = sc + (correction ? correction[e] : 0.f);
+    }
+    wave_sync();
+  }
   // lane j keeps the j-th choice (top <= 32 lanes of the 64)
   float my_pick = 0.f;
   int my_choice = 0;
@@ -103,7 +127,7 @@ moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const
     float best = -INFINITY;
     int at = 0x7fffffff;
     for (int e = lane; e < E; e += TS_WAVE) {
-      const float c = c_s[r * E + e];
+      const float c = c_s[e];
       if (c > best) { best = c; at = e; }                 // (ascending e: the lower index wins a tie)
     }
 #pragma unroll
@@ -113,9 +137,9 @@ moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const
       if (ob > best || (ob == best && oa < at)) { best = ob; at = oa; }
     }
     if (at >= E) at = j;                                  // (scores that are no numbers: still valid indices)
-    if (lane == j) { my_choice = at; my_pick = s_s[r * E + at]; }
+    if (lane == j) { my_choice = at; my_pick = s_s[at]; }
     wave_sync();
-    if (lane == 0) c_s[r * E + at] = -INFINITY;
+    if (lane == 0) c_s[at] = -INFINITY;
     wave_sync();
   }
   if (softmax_chosen) {                                   // the chosen logits' softmax: the first choice is the largest
@@ -132,17 +156,19 @@ moe_route_kernel(int32_t* __restrict__ ids_out, float* __restrict__ w_out, const
 
 extern "C" int ts_moe_route(int32_t* ids_out, float* w_out, const void* x, int x_dtype, const float* router,
                             const float* correction, int num_tokens, int K, int E, int top, float scale, int normalize,
-                            int softmax_chosen, hipStream_t stream) {
+                            int scoring, int extras, float* extra_out, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
-  if (K <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > MOE_MAX_TOP || top > E) return TS_BAD_SHAPE;
+  if (K <= 0 || E <= 0 || E > MOE_MAX_EXPERTS || top <= 0 || top > MOE_MAX_TOP || top > E || scoring < 0 || scoring > 2 ||
+      extras < 0 || extras > TS_WAVE || (extras && !extra_out))
+    return TS_BAD_SHAPE;
   const unsigned blocks = (num_tokens + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS;
-  const size_t lds = (size_t)MOE_ROUTE_TOKENS * (2 * E + MOE_ROUTE_CHUNK) * sizeof(float);
+  const size_t lds = (size_t)MOE_ROUTE_TOKENS * (2 * (E + extras) + MOE_ROUTE_CHUNK) * sizeof(float);
   if (x_dtype == 0)
     moe_route_kernel<float><<<blocks, MOE_ROUTE_THREADS, lds, stream>>>(ids_out, w_out, (const float*)x, router, correction,
-                                                                        num_tokens, K, E, top, scale, normalize, softmax_chosen);
+                                                                        num_tokens, K, E, top, scale, normalize, scoring, extras, extra_out);
   else if (x_dtype == 1)
     moe_route_kernel<bf16_t><<<blocks, MOE_ROUTE_THREADS, lds, stream>>>(ids_out, w_out, (const bf16_t*)x, router, correction,
-                                                                         num_tokens, K, E, top, scale, normalize, softmax_chosen);
+                                                                         num_tokens, K, E, top, scale, normalize, scoring, extras, extra_out);
   else return TS_BAD_DTYPE;
   return ts_check_launch();
 }
@@ -157,7 +183,8 @@ moe_group_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ sorted, 
   __shared__ int tile_s[MOE_MAX_EXPERTS + 1];
   for (int e = threadIdx.x; e < E; e += MOE_GROUP_THREADS) count_s[e] = 0;
   __syncthreads();
-  for (int p = threadIdx.x; p < P; p += MOE_GROUP_THREADS) atomicAdd(&count_s[ids[p]], 1);
+  for (int p = threadIdx.x; p < P; p += MOE_GROUP_THREADS)
+    if (ids[p] < E) atomicAdd(&count_s[ids[p]], 1);          // (a choice beyond the experts with matrices: an identity expert, in no tile)
   __syncthreads();
   if (threadIdx.x == 0) {
     int first = 0, tile = 0;
@@ -191,7 +218,7 @@ moe_group_kernel(const int32_t* __restrict__ ids, int32_t* __restrict__ sorted, 
   __syncthreads();
   for (int p = threadIdx.x; p < P; p += MOE_GROUP_THREADS) {
     const int e = ids[p];
-    sorted[first_s[e] + atomicAdd(&count_s[e], 1)] = p;
+    if (e < E) sorted[first_s[e] + atomicAdd(&count_s[e], 1)] = p;
   }
 }
 
@@ -674,10 +701,11 @@ extern "C" int ts_moe_gemm(void* out, int out_dtype, const void* x, int x_dtype,
 
 // A thread per four columns of a token (or per column, where rows are no whole 16-byte pieces): a step of one token
 // spreads over the row's width and waits for memory once.
-template <int VEC>
+template <int VEC, typename TX>
 __global__ void __launch_bounds__(MOE_THREADS)
 moe_combine_kernel(float* __restrict__ out, const float* __restrict__ rows, const float* __restrict__ weights,
-                   const float* __restrict__ shared, int width, int top) {
+                   const float* __restrict__ shared, int width, int top, const int32_t* __restrict__ ids, int real,
+                   const TX* __restrict__ x, const float* __restrict__ shared_gate) {
   const int64_t t = blockIdx.x;
   const int i = (blockIdx.y * MOE_THREADS + threadIdx.x) * VEC;
   if (i >= width) return;
@@ -686,6 +714,11 @@ moe_combine_kernel(float* __restrict__ out, const float* __restrict__ rows, cons
   for (int c = 0; c < VEC; ++c) acc[c] = 0.f;
   for (int j = 0; j < top; ++j) {
     const float w = weights[t * top + j];
+    if (ids && ids[t * top + j] >= real) {                // an identity expert: the token's input itself
+#pragma unroll
+      for (int c = 0; c < VEC; ++c) acc[c] = fmaf(w, Num<TX>::ld(x + t * width + i + c), acc[c]);
+      continue;
+    }
     const float* row = rows + (t * top + j) * width + i;
     if constexpr (VEC == 4) {
       const float4 v = *(const float4*)row;
@@ -694,27 +727,35 @@ moe_combine_kernel(float* __restrict__ out, const float* __restrict__ rows, cons
       acc[0] = fmaf(w, row[0], acc[0]);
     }
   }
+  const float g = shared_gate ? shared_gate[t] : 1.0f;
   if constexpr (VEC == 4) {
     if (shared) {
       const float4 v = *(const float4*)(shared + t * width + i);
-      acc[0] += v.x; acc[1] += v.y; acc[2] += v.z; acc[3] += v.w;
+      acc[0] = fmaf(g, v.x, acc[0]); acc[1] = fmaf(g, v.y, acc[1]); acc[2] = fmaf(g, v.z, acc[2]); acc[3] = fmaf(g, v.w, acc[3]);
     }
     *(float4*)(out + t * width + i) = make_float4(acc[0], acc[1], acc[2], acc[3]);
   } else {
-    if (shared) acc[0] += shared[t * width + i];
+    if (shared) acc[0] = fmaf(g, shared[t * width + i], acc[0]);
     out[t * width + i] = acc[0];
   }
 }
 
 extern "C" int ts_moe_combine(float* out, const float* rows, const float* weights, const float* shared, int num_tokens,
-                              int width, int top, hipStream_t stream) {
+                              int width, int top, const int32_t* ids, int real, const void* x, int x_dtype,
+                              const float* shared_gate, hipStream_t stream) {
   if (num_tokens <= 0) return TS_OK;
-  if (width <= 0 || top <= 0) return TS_BAD_SHAPE;
+  if (width <= 0 || top <= 0 || (ids && !x) || (shared_gate && !shared)) return TS_BAD_SHAPE;
+  if (x_dtype != 0 && x_dtype != 1) return TS_BAD_DTYPE;
   const bool by4 = width % 4 == 0 && (((uintptr_t)out | (uintptr_t)rows | (uintptr_t)shared) & 15) == 0;
   const int per_block = MOE_THREADS * (by4 ? 4 : 1);
   dim3 grid(num_tokens, (width + per_block - 1) / per_block);
   if (grid.y > 65535) return TS_BAD_SHAPE;
-  if (by4) moe_combine_kernel<4><<<grid, MOE_THREADS, 0, stream>>>(out, rows, weights, shared, width, top);
-  else moe_combine_kernel<1><<<grid, MOE_THREADS, 0, stream>>>(out, rows, weights, shared, width, top);
+#define MOE_COMBINE(VEC, TX) \
+  moe_combine_kernel<VEC, TX><<<grid, MOE_THREADS, 0, stream>>>(out, rows, weights, shared, width, top, ids, real, (const TX*)x, shared_gate)
+  if (by4 && x_dtype == 0) MOE_COMBINE(4, float);
+  else if (by4) MOE_COMBINE(4, bf16_t);
+  else if (x_dtype == 0) MOE_COMBINE(1, float);
+  else MOE_COMBINE(1, bf16_t);
+#undef MOE_COMBINE
   return ts_check_launch();
 }

@@ -178,12 +178,13 @@ extern "C" int ts_stream_update_norm(float* x, const void* a, int a_dtype, const
   return ts_check_launch();
 }
 
-// out[t, i] = act(in[t, i] + bias[i]); act 0: none, 1: relu squared, 2: gelu (tanh form), 3: silu
+// out[t, i] = act(in[t, i] + bias[i]); act 0: none, 1: relu squared, 2: gelu (tanh form), 3: silu, 4: tanh
 static __device__ __forceinline__ float rs_activate(float z, int act) {
   switch (act) {
     case 1: { const float r = fmaxf(z, 0.f); return r * r; }
     case 2: return 0.5f * z * (1.0f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
     case 3: return z / (1.0f + expf(-z));
+    case 4: return tanhf(z);
     default: return z;
   }
 }
@@ -227,7 +228,7 @@ bias_activation_by4_kernel(TO* __restrict__ out, const float* __restrict__ in, c
 extern "C" int ts_bias_activation(void* out, int out_dtype, const void* in, int in_dtype, const void* bias, int bias_dtype,
                                   int num_rows, int width, int act, hipStream_t stream) {
   if (num_rows <= 0) return TS_OK;
-  if (width <= 0 || act < 0 || act > 3) return TS_BAD_SHAPE;
+  if (width <= 0 || act < 0 || act > 4) return TS_BAD_SHAPE;
   for (int code : {out_dtype, in_dtype, bias_dtype})
     if (code != 0 && code != 1) return TS_BAD_DTYPE;
   const int64_t total = (int64_t)num_rows * width;
@@ -247,5 +248,83 @@ extern "C" int ts_bias_activation(void* out, int out_dtype, const void* in, int 
   if (blocks > 16384) blocks = 16384;
   bias_activation_kernel<<<(unsigned)blocks, RS_THREADS, 0, stream>>>(out, out_dtype, in, in_dtype, bias, bias_dtype, total,
                                                                      width, act);
+  return ts_check_launch();
+}
+
+// ---- a branch that passes an RMS norm of its own (and a learned scale per channel) before it is added ----
+// Row r: x[r] += a[r] / sqrt(mean(a[r]^2) + post_eps) * post_w * scale   (scale may be absent),
+// then, if asked for, h[r] = x[r] / sqrt(mean(x[r]^2) + eps) * w (the next norm), or h[r] = x[r] itself (w absent),
+// rounded to h's storage type at the store. A workgroup a row; every sum is taken by the same tree whatever the batch.
+__global__ void __launch_bounds__(RS_THREADS)
+stream_post_norm_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ post_w,
+                        const float* __restrict__ scale, float post_eps, void* __restrict__ h, int h_code,
+                        const float* __restrict__ w, float eps, int width) {
+  __shared__ float scratch[RS_THREADS / TS_WAVE];
+  const int64_t r = blockIdx.x;
+  float* xr = x + r * width;
+  const float* ar = a + r * width;
+  float squares = 0.f;
+  for (int i = threadIdx.x; i < width; i += RS_THREADS) squares = fmaf(ar[i], ar[i], squares);
+  const float inv_a = 1.0f / sqrtf(block_sum(squares, scratch) / (float)width + post_eps);
+  squares = 0.f;
+  for (int i = threadIdx.x; i < width; i += RS_THREADS) {
+    float add = ar[i] * inv_a * post_w[i];
+    if (scale) add *= scale[i];
+    const float v = xr[i] + add;
+    xr[i] = v;
+    squares = fmaf(v, v, squares);
+  }
+  if (!h) return;
+  float inv = 1.0f;
+  if (w) inv = 1.0f / sqrtf(block_sum(squares, scratch) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += RS_THREADS)      // (this thread's own elements, as it has just written them)
+    rs_store(h, h_code, r * width + i, w ? xr[i] * inv * w[i] : xr[i]);
+}
+
+extern "C" int ts_stream_post_norm(float* x, const float* a, const float* post_w, const float* scale, float post_eps, void* h,
+                                   int h_dtype, const float* w, float eps, int num_rows, int width, hipStream_t stream) {
+  if (num_rows <= 0) return TS_OK;
+  if (width <= 0 || !x || !a || !post_w) return TS_BAD_SHAPE;
+  if (h_dtype != 0 && h_dtype != 1) return TS_BAD_DTYPE;
+  stream_post_norm_kernel<<<num_rows, RS_THREADS, 0, stream>>>(x, a, post_w, scale, post_eps, h, h_dtype, w, eps, width);
+  return ts_check_launch();
+}
+
+// out = sa * a + sb * b, element by element (what two mixers side by side have made, each with its own factor)
+__global__ void __launch_bounds__(RS_THREADS)
+scaled_sum_kernel(float* __restrict__ out, const float* __restrict__ a, float sa, const float* __restrict__ b, float sb, int64_t total) {
+  for (int64_t i = (int64_t)blockIdx.x * RS_THREADS + threadIdx.x; i < total; i += (int64_t)gridDim.x * RS_THREADS)
+    out[i] = fmaf(sb, b[i], sa * a[i]);
+}
+
+extern "C" int ts_scaled_sum(float* out, const float* a, float sa, const float* b, float sb, int64_t total, hipStream_t stream) {
+  if (total <= 0) return TS_OK;
+  int64_t blocks = (total + RS_THREADS - 1) / RS_THREADS;
+  if (blocks > 16384) blocks = 16384;
+  scaled_sum_kernel<<<(unsigned)blocks, RS_THREADS, 0, stream>>>(out, a, sa, b, sb, total);
+  return ts_check_launch();
+}
+
+// out[t, j] = act(sums[t, j]) * table[ids[t], offset + j]: a gate's sums times a stretch of a token's row of a table
+__global__ void __launch_bounds__(RS_THREADS)
+gather_gate_kernel(void* __restrict__ out, int out_code, const float* __restrict__ sums, const void* __restrict__ table,
+                   int table_code, int64_t table_stride, int offset, const int32_t* __restrict__ ids, int64_t total, int width, int act) {
+  for (int64_t idx = (int64_t)blockIdx.x * RS_THREADS + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * RS_THREADS) {
+    const int64_t t = idx / width;
+    const int j = (int)(idx - t * width);
+    rs_store(out, out_code, idx, rs_activate(sums[idx], act) * rs_load(table, table_code, (int64_t)ids[t] * table_stride + offset + j));
+  }
+}
+
+extern "C" int ts_gather_gate(void* out, int out_dtype, const float* sums, const void* table, int table_dtype, int64_t table_stride,
+                              int offset, const int32_t* ids, int num_rows, int width, int act, hipStream_t stream) {
+  if (num_rows <= 0) return TS_OK;
+  if (width <= 0 || offset < 0 || table_stride < offset + width || act < 0 || act > 4) return TS_BAD_SHAPE;
+  if ((out_dtype | table_dtype) & ~1) return TS_BAD_DTYPE;
+  const int64_t total = (int64_t)num_rows * width;
+  int64_t blocks = (total + RS_THREADS - 1) / RS_THREADS;
+  if (blocks > 16384) blocks = 16384;
+  gather_gate_kernel<<<(unsigned)blocks, RS_THREADS, 0, stream>>>(out, out_dtype, sums, table, table_dtype, table_stride, offset, ids,
+                                                                 total, width, act);
   return ts_check_launch();
 }

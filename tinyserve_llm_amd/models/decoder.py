@@ -42,7 +42,8 @@ class DecoderModel:
             self.layers.append(Layer(
                 mixer=base.make("mixer", ls.mixer), feed_forward=base.make("feed_forward", ls.feed_forward),
                 norms={name: base.make("norm", ps) for name, ps in ls.norms.items()}, block=ls.block,
-                block_args=dict(ls.block_args)))
+                block_args=dict(ls.block_args),
+                token_inputs={name: base.make("token_input", ps) for name, ps in ls.token_inputs.items()}))
         self.final_norm = base.make("norm", spec.final_norm)
         self.position_encodings = {name: base.make("position_encoding", ps)
                                    for name, ps in spec.position_encodings.items()}
@@ -130,6 +131,8 @@ class DecoderModel:
         for i, layer in enumerate(self.layers):
             for part_name, part in layer.parts().items():
                 part.bind(grouped.get(f"layers.{i}.{part_name}", {}))
+            for part in layer.token_inputs.values():
+                part.attach(self.embedding.side_table())
         for name, enc in self.position_encodings.items():
             enc.bind(grouped.get(f"positions.{name}", {}))
             enc.prepare(device)

@@ -28,6 +28,9 @@ class Architecture:
     config_to_dict: Callable[[Any], Mapping[str, Any]] | None = None
     # The class of the typed configuration; None: the class whose classmethod `config_from_dict` is.
     config_type: type | None = None
+    # Sizes that config.json leaves to the checkpoint: (configuration, {tensor name: shape}) -> configuration.
+    # `read_config` calls it with the shapes of the folder's tensors (their files' headers; no tensor is read).
+    sizes_from_checkpoint: Callable[[Any, Mapping[str, tuple]], Any] | None = None
 
     def owns(self, config: Any) -> bool:
         """Whether `config` is a typed configuration of this architecture."""
@@ -100,4 +103,20 @@ def read_config(folder: str) -> tuple[Architecture, Any]:
     with open(path) as f:
         raw = json.load(f)
     arch = resolve(raw)
-    return arch, arch.config_from_dict(raw)
+    config = arch.config_from_dict(raw)
+    if arch.sizes_from_checkpoint is not None:
+        config = arch.sizes_from_checkpoint(config, checkpoint_shapes(folder))
+    return arch, config
+
+
+def checkpoint_shapes(folder: str) -> dict[str, tuple]:
+    """{tensor name: shape} of a folder's model*.safetensors files, from their headers."""
+    from glob import glob
+
+    from safetensors import safe_open
+    shapes: dict[str, tuple] = {}
+    for file in sorted(glob(os.path.join(folder, "model*.safetensors"))):
+        with safe_open(file, "pt", "cpu") as f:
+            for name in f.keys():
+                shapes[name] = tuple(f.get_slice(name).get_shape())
+    return shapes

@@ -21,6 +21,8 @@ class LayerSpec:
     norms: Mapping[str, PartSpec]
     block: str = "pre_norm"
     block_args: Mapping[str, object] = field(default_factory=dict)      # constants of the arrangement itself
+    # parts of the "token_input" family by the names the arrangement looks them up under (and their parameters are known by)
+    token_inputs: Mapping[str, PartSpec] = field(default_factory=dict)
 
     @classmethod
     def pre_norm(cls, mixer: PartSpec, feed_forward: PartSpec, mixer_norm: PartSpec, ff_norm: PartSpec) -> "LayerSpec":

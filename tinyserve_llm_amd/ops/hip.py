@@ -89,11 +89,11 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_dyt": [p, i, p, i, p, i, p, i, p, p, p, p, i, i, p],
         "ts_dyt_stream": [p, p, i, p, p, p, p, i, p, p, p, i, i, p],
         "ts_embedding_dyt_stream": [p, p, i, p, f, p, p, p, i, i, p],
-        "ts_capped_glu": [p, i, p, i, i64, i, i, f, f, f, p],
+        "ts_capped_glu": [p, i, p, i, i64, i, i, f, f, f, i, p],
         "ts_conv_finish": [p, p, p, p, i64, p, p, p, p, f, p, p, p, p, p, i, i, i, i, i, i, f, i, i, i64, i64, i64, i64, i64,
                            i64, i64, i, i, i, p],
         "ts_conv_state_update": [p, p, i64, p, p, i, i, i, i, p],
-        "ts_moe_route": [p, p, p, i, p, p, i, i, i, i, f, i, i, p],
+        "ts_moe_route": [p, p, p, i, p, p, i, i, i, i, f, i, i, i, p, p],
         "ts_moe_group": [p, p, p, i, i, i, i, p],
         "ts_moe_gemm": [p, i, p, i, p, p, p, i, i, i, i, i, i, f, f, f, i, p],
         "ts_segment_rmsnorm": [p, i, i64, p, i64, i, p, f, i, p],
@@ -102,13 +102,20 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_latent_mfma_takes": [i, i],
         "ts_heads_gemm_mfma": [p, i, i64, i64, p, i, i64, i64, p, i64, i64, i, i, i, i, p, i64, p],
         "ts_paged_attention_latent_mfma": [p, i, p, p, p, p, p, p, p, i, i, i, i, i, i, i, i64, i64, i64, i64, i64, i, f, i, i, i, p, p, p],
-        "ts_rotate_heads": [p, i, i64, i64, p, i64, i64, i, i, i, p, f, p, i, p],
+        "ts_rotate_heads": [p, i, i64, i64, p, i, i64, i64, i, i, i, p, f, p, i, i, p, i64, p],
         "ts_heads_gemm": [p, i, i64, i64, p, i, i64, i64, p, i, i64, i64, i64, i, i, i, i, p, i64, p],
         "ts_paged_attention_latent": [p, i, p, i, p, i, p, p, p, i, i, i, i, i, i64, i64, i, f, i, i, p],
         "ts_mlstm_scan": [p, p, i64, p, p, p, p, p, i, i, i, i, i, f, f, p],
         "ts_mlstm_scan_chunks": [p, p, i64, p, p, p, p, p, p, p, p, p, i, i, i, i, i, f, f, p],
-        "ts_mlstm_finish": [p, i, p, p, p, i64, i, i, i, f, p],
-        "ts_moe_combine": [p, p, p, p, i, i, i, p],
+        "ts_mlstm_finish": [p, i, p, p, p, i64, i, i, i, f, i, i, p],
+        "ts_moe_combine": [p, p, p, p, i, i, i, p, i, p, i, p, p],
+        "ts_decay_scan": [p, p, i64, p, i64, p, i64, p, i64, p, p, p, i64, p, p, i, i, i, i, i, f, f, i, i, p],
+        "ts_token_shift": [p, p, i, p, p, i64, p, p, p, i, i, i, p],
+        "ts_token_shift_keep": [p, i64, p, i, p, p, i, i, p],
+        "ts_stream_post_norm": [p, p, p, p, f, p, i, p, f, i, i, p],
+        "ts_scaled_sum": [p, p, f, p, f, i64, p],
+        "ts_gather_gate": [p, i, p, p, i, i64, i, p, i, i, i, p],
+        "ts_qkv_prepare": [p, p, i, i, i, i, i, p, p, f, p, i, p],
         "ts_gemm_skinny_rope_bf16": [p, p, p, p, p, p, i, i, i64, i64, f, i, i, p, p, p, p, p, i, i, i, i, i, i64, i64, i64,
                                      i64, i64, i64, i64, p, i, p],
     }
@@ -1509,7 +1516,7 @@ def linear_bf16(x: torch.Tensor, weight: torch.Tensor, out_dtype: torch.dtype = 
         return gemm_rows64(x, packed.by16, out_dtype)
     if _many_rows == "tiled" and tiled_takes(x, weight):
         return gemm_tiled(x, weight, out_dtype=out_dtype)
-    if x.shape[1] % 8 or x.stride(0) % 8 or weight.stride(0) % 8:
+    if x.shape[1] % 8 or x.stride(0) % 8 or weight.stride(0) % 8 or weight.shape[0] < 8:
         # rows that are no whole 16-byte pieces: the library has no algorithm for every such shape; the
         # exact kernel takes any (32-bit multiply-adds, slower, for sizes no real model has)
         return gemm_exact(x, weight, out_dtype)
@@ -1659,7 +1666,7 @@ def stream_update_norm(x: torch.Tensor, a: torch.Tensor | None = None, b: torch.
     return outs[0], outs[1]
 
 
-ACTIVATIONS = {"none": 0, "relu2": 1, "gelu_tanh": 2, "silu": 3}
+ACTIVATIONS = {"none": 0, "relu2": 1, "gelu_tanh": 2, "silu": 3, "tanh": 4}
 
 
 def bias_activation(x: torch.Tensor, bias: torch.Tensor | None, activation: str, out_dtype: torch.dtype) -> torch.Tensor:
@@ -1888,16 +1895,18 @@ def embedding_dyt_stream(table: torch.Tensor, ids: torch.Tensor, scale: float = 
     return out
 
 
-def capped_glu(gate_up: torch.Tensor, limit: float, slope: float, up_shift: float, out_dtype: torch.dtype) -> torch.Tensor:
+def capped_glu(gate_up: torch.Tensor, limit: float, slope: float, up_shift: float, out_dtype: torch.dtype,
+               relu: bool = False) -> torch.Tensor:
     """From rows [gate | up] (float32 or `out_dtype`): g = min(gate, limit), u = clamp(up, -limit, limit)
-    (limit <= 0: no cap), y = g sigmoid(slope g) (u + up_shift), in 32-bit, stored as `out_dtype`."""
+    (limit <= 0: no cap), y = g sigmoid(slope g) (u + up_shift), or max(g, 0) (u + up_shift) with `relu`, in 32-bit,
+    stored as `out_dtype`."""
     _gpu(gate_up)
     _need(gate_up.dim() == 2 and gate_up.shape[1] % 2 == 0 and gate_up.stride(1) == 1 and gate_up.stride(0) >= gate_up.shape[1],
           "the input must be [tokens, 2 ff] with contiguous rows")
     n, ff = gate_up.shape[0], gate_up.shape[1] // 2
     out = torch.empty((n, ff), dtype=out_dtype, device=gate_up.device)
     _run("capped_glu", library().ts_capped_glu(_ptr(out), _code(out_dtype), _ptr(gate_up), _code(gate_up.dtype), gate_up.stride(0),
-                                               n, ff, float(limit), float(slope), float(up_shift), _stream()))
+                                               n, ff, float(limit), float(slope), float(up_shift), int(relu), _stream()))
     return out
 
 
@@ -1990,23 +1999,28 @@ MOE_MAX_TOP = 32
 
 
 def moe_route(x: torch.Tensor, router: torch.Tensor, correction: torch.Tensor | None, top: int, scale: float,
-              normalize: bool = True, softmax_chosen: bool = False) -> tuple[torch.Tensor, torch.Tensor]:
+              normalize: bool = True, softmax_chosen: bool = False, softmax_all: bool = False, extras: int = 0):
     """(experts int32 [tokens, top], weights float32 [tokens, top]): scores s = sigmoid(x · routerᵀ) in 32-bit;
     the `top` experts with the largest s + correction; weights s of the chosen, over their sum (+ 1e-20) if
     `normalize`, times `scale`. `softmax_chosen`: the logits themselves are the scores, and the weights are the
-    softmax over the chosen experts' logits alone (times `scale`)."""
+    softmax over the chosen experts' logits alone (times `scale`). `softmax_all`: the scores are the softmax over
+    all the experts' logits. `extras`: the router's last rows beyond the experts, whose logits' sigmoids come back as
+    a third result, float32 [tokens, extras] (a gate on a shared expert, say)."""
     _gpu(x, router, correction)
     _need(x.dim() == 2 and x.is_contiguous(), "the input must be contiguous [tokens, width]")
-    E = router.shape[0]
-    _need(router.dtype == torch.float32 and router.shape == (E, x.shape[1]) and router.is_contiguous(), "the router must be float32 [experts, width]")
+    _need(0 <= extras < router.shape[0] and extras <= 64 and not (softmax_chosen and softmax_all), "up to 64 extra rows; one way of scoring")
+    E = router.shape[0] - extras
+    _need(router.dtype == torch.float32 and router.shape == (E + extras, x.shape[1]) and router.is_contiguous(), "the router must be float32 [experts, width]")
     _need(correction is None or (correction.dtype == torch.float32 and correction.shape == (E,) and correction.is_contiguous()),
           "the correction must be float32 [experts]")
     _need(1 <= top <= min(E, MOE_MAX_TOP) and E <= MOE_MAX_EXPERTS, lambda: f"1 <= top <= min(experts, {MOE_MAX_TOP}), experts <= {MOE_MAX_EXPERTS}")
     ids = torch.empty((x.shape[0], top), dtype=torch.int32, device=x.device)
     weights = torch.empty((x.shape[0], top), dtype=torch.float32, device=x.device)
+    extra = torch.empty((x.shape[0], extras), dtype=torch.float32, device=x.device) if extras else None
     _run("moe_route", library().ts_moe_route(_ptr(ids), _ptr(weights), _ptr(x), _code(x.dtype), _ptr(router), _ptr(correction),
-                                             x.shape[0], x.shape[1], E, top, float(scale), int(normalize), int(softmax_chosen), _stream()))
-    return ids, weights
+                                             x.shape[0], x.shape[1], E, top, float(scale), int(normalize),
+                                             2 if softmax_all else int(softmax_chosen), extras, _ptr(extra), _stream()))
+    return (ids, weights, extra) if extras else (ids, weights)
 
 
 class ExpertTiles:
@@ -2028,7 +2042,8 @@ def moe_tile_rows(pairs: int, experts: int, dtype: torch.dtype, k_sizes: "tuple[
 
 
 def moe_group(ids: torch.Tensor, experts: int, tile_rows: int = MOE_TILE_ROWS) -> ExpertTiles:
-    """Groups the step's pairs by expert and cuts the groups into tiles of up to `tile_rows` rows."""
+    """Groups the step's pairs by expert and cuts the groups into tiles of up to `tile_rows` rows. A pair whose choice is
+    `experts` or beyond (an identity expert, which has no matrices) lands in no tile."""
     _gpu(ids)
     _need(tile_rows in (MOE_TILE_ROWS, MOE_WIDE_TILE_ROWS, MOE_LDS_TILE_ROWS), "tiles of 16, 64 or 128 rows")
     _need(ids.dtype == torch.int32 and ids.dim() == 2 and ids.is_contiguous(), "the chosen experts must be contiguous int32 [tokens, top]")
@@ -2070,16 +2085,28 @@ def moe_gemm(x: torch.Tensor, weights: torch.Tensor, grouped: ExpertTiles, out_d
     return out
 
 
-def moe_combine(rows: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None = None) -> torch.Tensor:
-    """out[t] = sum_j weights[t, j] * rows[t * top + j] (+ shared[t]), float32."""
-    _gpu(rows, weights, shared)
+def moe_combine(rows: torch.Tensor, weights: torch.Tensor, shared: torch.Tensor | None = None, *,
+                identity: "tuple[torch.Tensor, int, torch.Tensor] | None" = None, shared_gate: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = sum_j weights[t, j] * rows[t * top + j] (+ shared[t]), float32. `identity` = (the chosen experts int32
+    [tokens, top], the number of experts with matrices, the experts' input [tokens, width]): a choice at or beyond that
+    number stands for an expert that hands its input through, and its row is the token's input. `shared_gate` (float32
+    [tokens] or [tokens, 1]): the shared rows are multiplied by it, a number per token."""
+    _gpu(rows, weights, shared, shared_gate)
     T, top = weights.shape
+    ids, real, x = identity if identity is not None else (None, 0, None)
+    if identity is not None:
+        _gpu(ids, x)
+        _need(ids.dtype == torch.int32 and ids.shape == (T, top) and ids.is_contiguous(), "the chosen experts must be contiguous int32 [tokens, top]")
+        _need(x.shape == (T, rows.shape[1]) and x.is_contiguous() and x.dtype in _DTYPE_CODE, "the experts' input must be contiguous [tokens, width]")
+    _need(shared_gate is None or (shared is not None and shared_gate.dtype == torch.float32 and shared_gate.numel() == T and shared_gate.is_contiguous()),
+          "the shared expert's gate is float32, a number per token")
     _need(rows.dtype == torch.float32 and rows.dim() == 2 and rows.shape[0] == T * top and rows.is_contiguous(), "rows must be contiguous float32 [tokens * top, width]")
     _need(weights.dtype == torch.float32 and weights.is_contiguous(), "weights must be contiguous float32 [tokens, top]")
     _need(shared is None or (shared.dtype == torch.float32 and shared.shape == (T, rows.shape[1]) and shared.is_contiguous()),
           "the shared rows must be contiguous float32 [tokens, width]")
     out = torch.empty((T, rows.shape[1]), dtype=torch.float32, device=rows.device)
-    _run("moe_combine", library().ts_moe_combine(_ptr(out), _ptr(rows), _ptr(weights), _ptr(shared), T, rows.shape[1], top, _stream()))
+    _run("moe_combine", library().ts_moe_combine(_ptr(out), _ptr(rows), _ptr(weights), _ptr(shared), T, rows.shape[1], top, _ptr(ids), int(real),
+                                                 _ptr(x), 0 if x is None else _code(x.dtype), _ptr(shared_gate), _stream()))
     return out
 
 
@@ -2172,20 +2199,23 @@ def latent_finish(down: torch.Tensor, q_off: int, q_rank: int, kv_off: int, rank
 
 
 def rotate_heads(dst: torch.Tensor, src: torch.Tensor, freqs: torch.Tensor, amplitude: float, positions: torch.Tensor,
-                 interleaved: bool = True) -> None:
+                 interleaved: bool = True, back: bool = False, gate: torch.Tensor | None = None) -> None:
     """dst[t, h, :rot] = src[t, h, :rot] turned by positions[t] (rot = 2 len(freqs); pairs (2i, 2i+1) if `interleaved`,
-    else (i, i + rot/2); cosine and sine times `amplitude`). `src` float32 and `dst` are views [tokens, heads, >= rot]
-    whose last dimension is contiguous."""
-    _gpu(dst, src, freqs, positions)
+    else (i, i + rot/2); cosine and sine times `amplitude`), or turned back by as much with `back`. `src` (float32, or of
+    `dst`'s type) and `dst` are views [tokens, heads, >= rot] whose last dimension is contiguous; they may be the same.
+    `gate` (float32 [tokens, heads], rows may lie apart): what is turned is multiplied by sigmoid(gate[t, h])."""
+    _gpu(dst, src, freqs, positions, gate)
     T, H = src.shape[0], src.shape[1]
     rot = 2 * freqs.shape[0]
     _check_freqs(freqs, rot)
     _check_step_vectors(T, positions=positions)
-    _need(src.dtype == torch.float32 and src.dim() == 3 and dst.dim() == 3 and dst.shape[:2] == src.shape[:2]
+    _need(src.dtype in (torch.float32, dst.dtype) and src.dim() == 3 and dst.dim() == 3 and dst.shape[:2] == src.shape[:2]
           and src.shape[2] >= rot and dst.shape[2] >= rot and src.stride(2) == 1 and dst.stride(2) == 1, "views [tokens, heads, >= rot]")
+    _need(gate is None or (gate.dtype == torch.float32 and gate.shape == (T, H) and gate.stride(1) == 1), "the gate is float32 [tokens, heads]")
     _run("rotate_heads", library().ts_rotate_heads(
-        _ptr(dst), _code(dst.dtype), dst.stride(0), dst.stride(1), _ptr(src), src.stride(0), src.stride(1), H, rot, int(interleaved),
-        _ptr(freqs), float(amplitude), _ptr(positions), T, _stream()))
+        _ptr(dst), _code(dst.dtype), dst.stride(0), dst.stride(1), _ptr(src), _code(src.dtype), src.stride(0), src.stride(1), H, rot,
+        int(interleaved), _ptr(freqs), float(amplitude), _ptr(positions), T, int(back), _ptr(gate), 0 if gate is None else gate.stride(0),
+        _stream()))
 
 
 def heads_gemm_mfma_takes(x: torch.Tensor, w: torch.Tensor, out: torch.Tensor) -> bool:
@@ -2372,14 +2402,143 @@ def mlstm_scan(proj: torch.Tensor, i_bias: torch.Tensor, f_bias: torch.Tensor, s
     return out
 
 
-def mlstm_finish(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, heads: int, vdim: int, eps: float, out_dtype: torch.dtype) -> torch.Tensor:
+def mlstm_finish(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, heads: int, vdim: int, eps: float, out_dtype: torch.dtype,
+                 silu_gate: bool = False) -> torch.Tensor:
     """Each head's row of o (float32 [tokens, heads vdim]) divided by its root mean square, times `weight` (float32
-    [heads vdim]), times sigmoid(gate) (float32 [tokens, heads vdim], rows may lie apart), as `out_dtype`."""
+    [heads vdim], or [vdim]: one weight that all heads share), times sigmoid(gate) (float32 [tokens, heads vdim], rows
+    may lie apart; with `silu_gate` times gate sigmoid(gate)), as `out_dtype`."""
     _gpu(o, weight, gate)
     T = o.shape[0]
     _need(o.dtype == torch.float32 and o.shape == (T, heads * vdim) and o.is_contiguous(), "o must be contiguous float32 [tokens, heads vdim]")
-    _need(weight.dtype == torch.float32 and weight.shape == (heads * vdim,) and weight.is_contiguous(), "the weight must be float32 [heads vdim]")
+    _need(weight.dtype == torch.float32 and weight.shape in ((heads * vdim,), (vdim,)) and weight.is_contiguous(),
+          "the weight must be float32 [heads vdim], or [vdim] for all heads")
     out = torch.empty((T, heads * vdim), dtype=out_dtype, device=o.device)
     _run("mlstm_finish", library().ts_mlstm_finish(_ptr(out), _code(out_dtype), _ptr(o), _ptr(weight), _ptr(gate), _check_gate(gate, T, heads * vdim),
-                                                   T, heads, vdim, float(eps), _stream()))
+                                                   T, heads, vdim, float(eps), vdim if weight.shape[0] == heads * vdim else 0, int(silu_gate),
+                                                   _stream()))
     return out
+
+
+# ---- linear attention with a decay per key channel; token shift; what a sandwiched RMS norm needs ----
+
+DECAY_FORMS = {"sigmoid_root": 0, "double_exponent": 1}
+DECAY_MAX_DIM = 1024
+DECAY_FULL_WORKGROUPS = 512      # workgroups of four waves from which a step keeps them (fewer: one wave each, four times as many)
+
+
+def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, z_bias: torch.Tensor, state: torch.Tensor,
+               cu_seqlens: torch.Tensor, state_slots: torch.Tensor, heads: int, dim: int, vdim: int, *, form: str, tau: float = 1.0,
+               q_scale: float = 1.0, bonus: torch.Tensor | None = None) -> torch.Tensor:
+    """Linear attention with a decay per key channel over a packed step. q, k, z float32 [tokens, heads dim] and v
+    float32 [tokens, heads vdim] are views whose rows may lie apart (columns of fused projections); z_bias float32
+    [heads dim]. The decays are w = sigmoid(z + z_bias)^(1 / tau) (`form` "sigmoid_root") or exp(-exp(z + z_bias))
+    ("double_exponent"). Without `bonus`: S <- diag(w) S + k v^T, o = S^T (q q_scale). With `bonus` (float32 [heads, dim]):
+    o = (S + diag(bonus) k v^T)^T q first, then the same update. `state` float32 [slots, >= heads dim vdim]: each
+    request's S lies at the start of its slot's row, is read there and written back. Returns o float32 [tokens, heads vdim]."""
+    _gpu(q, k, v, z, z_bias, state, cu_seqlens, state_slots, bonus)
+    T = q.shape[0]
+    _need(form in DECAY_FORMS, lambda: f"form {form!r}: one of {sorted(DECAY_FORMS)}")
+    for name, t, width in (("q", q, heads * dim), ("k", k, heads * dim), ("z", z, heads * dim), ("v", v, heads * vdim)):
+        _need(t.dtype == torch.float32 and t.shape == (T, width) and t.stride(1) == 1 and t.stride(0) >= width,
+              lambda: f"{name} must be float32 [tokens, {width}] with contiguous rows")
+    _need(z_bias.dtype == torch.float32 and z_bias.shape == (heads * dim,) and z_bias.is_contiguous(), "the decays' bias must be float32 [heads dim]")
+    _need(bonus is None or (bonus.dtype == torch.float32 and bonus.numel() == heads * dim and bonus.is_contiguous()), "the bonus must be float32 [heads, dim]")
+    _need(state.dtype == torch.float32 and state.dim() == 2 and state.shape[1] >= heads * dim * vdim and state.stride(1) == 1,
+          "the state must be float32 [slots, >= heads dim vdim]")
+    S = state_slots.shape[0]
+    _need(cu_seqlens.dtype == torch.int32 and cu_seqlens.shape == (S + 1,) and state_slots.dtype == torch.int32, "cu_seqlens int32 [requests + 1], slots int32 [requests]")
+    _need(0 < dim <= DECAY_MAX_DIM and tau > 0, lambda: f"heads of up to {DECAY_MAX_DIM} dimensions, a positive tau")
+    out = torch.empty((T, heads * vdim), dtype=torch.float32, device=q.device)
+    waves = 4 if vdim >= 64 and S * heads * (vdim // 64) >= DECAY_FULL_WORKGROUPS else 1
+    _run("decay_scan", library().ts_decay_scan(
+        _ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(z), z.stride(0), _ptr(z_bias), _ptr(bonus),
+        _ptr(state), state.stride(0), _ptr(cu_seqlens), _ptr(state_slots), S, heads, dim, vdim, DECAY_FORMS[form], float(tau),
+        float(q_scale), int(bonus is not None), waves, _stream()))
+    return out
+
+
+def token_shift(h: torch.Tensor, mu: torch.Tensor, kept: torch.Tensor, ctx) -> torch.Tensor:
+    """out[s, t] = h[t] + (h[t - 1] - h[t]) * mu[s] for every mix s (mu float32 [mixes, width]); for a request's first
+    token of the step h[t - 1] is the row that `kept` (float32 [slots, width], a view whose rows may lie apart) holds
+    at the request's state slot. Returns [mixes, tokens, width] of h's type. `token_shift_keep` leaves the step's last
+    rows in `kept` afterwards."""
+    _gpu(h, mu, kept)
+    T, W = h.shape
+    _need(h.dim() == 2 and h.is_contiguous(), "h must be contiguous [tokens, width]")
+    _need(mu.dtype == torch.float32 and mu.dim() == 2 and mu.shape[1] == W and mu.is_contiguous(), "mu must be float32 [mixes, width]")
+    _need(kept.dtype == torch.float32 and kept.dim() == 2 and kept.shape[1] == W and kept.stride(1) == 1, "the kept rows must be float32 [slots, width]")
+    out = torch.empty((mu.shape[0], T, W), dtype=h.dtype, device=h.device)
+    _run("token_shift", library().ts_token_shift(_ptr(out), _ptr(h), _code(h.dtype), _ptr(mu), _ptr(kept), kept.stride(0), _ptr(ctx.cu_seqlens),
+                                                 _ptr(ctx.seq_of_token), _ptr(ctx.state_slots), T, W, mu.shape[0], _stream()))
+    return out
+
+
+def token_shift_keep(kept: torch.Tensor, h: torch.Tensor, ctx) -> None:
+    """kept[slot of request s] = the last row of h that request s feeds in this step (nothing for a request that feeds none)."""
+    _gpu(h, kept)
+    _need(h.dim() == 2 and h.is_contiguous() and kept.dtype == torch.float32 and kept.dim() == 2 and kept.shape[1] == h.shape[1]
+          and kept.stride(1) == 1, "h contiguous [tokens, width], the kept rows float32 [slots, width]")
+    _run("token_shift_keep", library().ts_token_shift_keep(_ptr(kept), kept.stride(0), _ptr(h), _code(h.dtype), _ptr(ctx.cu_seqlens),
+                                                           _ptr(ctx.state_slots), ctx.state_slots.shape[0], h.shape[1], _stream()))
+
+
+def stream_post_norm(x: torch.Tensor, a: torch.Tensor, post_weight: torch.Tensor, scale: torch.Tensor | None, post_eps: float,
+                     weight: torch.Tensor | None = None, eps: float = 0.0, out_dtype: torch.dtype | None = None) -> torch.Tensor | None:
+    """The float32 stream x [tokens, width] takes x += a / sqrt(mean(a^2) + post_eps) * post_weight * scale in place (a
+    float32, what a branch has made; `scale` float32 [width] or None). With `out_dtype`, the updated rows come back in
+    that type: normalised and times `weight` (x / sqrt(mean(x^2) + eps) * weight), or as they are if `weight` is None."""
+    _gpu(x, a, post_weight, scale, weight)
+    _need(x.dtype == torch.float32 and x.dim() == 2 and x.is_contiguous() and a.dtype == torch.float32 and a.shape == x.shape and a.is_contiguous(),
+          "the stream and the branch's rows must be contiguous float32 [tokens, width]")
+    for w in (post_weight, scale, weight):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == (x.shape[1],) and w.is_contiguous()), "weights and scales must be float32 [width]")
+    _need(weight is None or out_dtype is not None, "a norm on the way out needs the rows' type")
+    out = torch.empty(x.shape, dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    _run("stream_post_norm", library().ts_stream_post_norm(_ptr(x), _ptr(a), _ptr(post_weight), _ptr(scale), float(post_eps), _ptr(out),
+                                                           0 if out is None else _code(out_dtype), _ptr(weight), float(eps), x.shape[0], x.shape[1], _stream()))
+    return out
+
+
+def scaled_sum(a: torch.Tensor, sa: float, b: torch.Tensor, sb: float) -> torch.Tensor:
+    """sa * a + sb * b, float32, element by element."""
+    _gpu(a, b)
+    _need(a.dtype == torch.float32 and b.dtype == torch.float32 and a.shape == b.shape and a.is_contiguous() and b.is_contiguous(),
+          "two contiguous float32 tensors of one shape")
+    out = torch.empty_like(a)
+    _run("scaled_sum", library().ts_scaled_sum(_ptr(out), _ptr(a), float(sa), _ptr(b), float(sb), a.numel(), _stream()))
+    return out
+
+
+def gather_gate(sums: torch.Tensor, table: torch.Tensor, offset: int, ids: torch.Tensor, activation: str, out_dtype: torch.dtype) -> torch.Tensor:
+    """out[t, j] = act(sums[t, j]) * table[ids[t], offset + j]: a gate's float32 sums [tokens, n] times a stretch of each
+    token's row of a table (ids int32, checked against the table on the host), as `out_dtype`."""
+    _gpu(sums, table, ids)
+    T, n = sums.shape
+    _need(activation in ACTIVATIONS, lambda: f"activation {activation!r}: one of {sorted(ACTIVATIONS)}")
+    _need(sums.dtype == torch.float32 and sums.is_contiguous(), "the sums must be contiguous float32 [tokens, n]")
+    _need(table.dim() == 2 and table.stride(1) == 1 and 0 <= offset and offset + n <= table.shape[1], "the stretch must lie inside the table's rows")
+    _need(ids.dtype == torch.int32 and ids.shape == (T,) and ids.is_contiguous(), "ids must be int32 [tokens]")
+    out = torch.empty((T, n), dtype=out_dtype, device=sums.device)
+    _run("gather_gate", library().ts_gather_gate(_ptr(out), _code(out_dtype), _ptr(sums), _ptr(table), _code(table.dtype), table.stride(0),
+                                                 int(offset), _ptr(ids), T, n, ACTIVATIONS[activation], _stream()))
+    return out
+
+
+def qkv_prepare(qkv: torch.Tensor, positions: torch.Tensor, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int, *,
+                q_weight: torch.Tensor | None = None, k_weight: torch.Tensor | None = None, eps: float = 0.0,
+                value_freqs: torch.Tensor | None = None, value_interleaved: bool = False) -> None:
+    """In place on the projected float32 rows q | k | v, before q and k turn: each q head (each k head) divided by its root
+    mean square and multiplied by `q_weight` (`k_weight`), float32 [head_dim], one weight for all heads; each value head
+    turned by the token's position over all its dimensions (`value_freqs` float64 [value_dim / 2]; pairs (m, m + value_dim/2),
+    or (2m, 2m + 1) with `value_interleaved`)."""
+    _gpu(qkv, positions, q_weight, k_weight, value_freqs)
+    T = qkv.shape[0]
+    row = (num_heads + num_kv_heads) * head_dim + num_kv_heads * value_dim
+    _need(qkv.dtype == torch.float32 and qkv.shape == (T, row) and qkv.is_contiguous(), lambda: f"qkv must be contiguous float32 [tokens, {row}]")
+    _check_step_vectors(T, positions=positions)
+    for w in (q_weight, k_weight):
+        _need(w is None or (w.dtype == torch.float32 and w.shape == (head_dim,) and w.is_contiguous()), "a head norm's weight is float32 [head_dim]")
+    if value_freqs is not None:
+        _check_freqs(value_freqs, value_dim)
+    _run("qkv_prepare", library().ts_qkv_prepare(_ptr(qkv), _ptr(positions), T, num_heads, num_kv_heads, head_dim, value_dim, _ptr(q_weight),
+                                                 _ptr(k_weight), float(eps), _ptr(value_freqs), int(value_interleaved), _stream()))

@@ -140,12 +140,22 @@ class GeneralAttention(Mixer):
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int, value_dim: int | None = None,
                  position: str | None = None, scale: float | None = None, softcap: float = 0.0, sink: bool = False,
                  qk_norm_eps: float | None = None, v_norm_eps: float | None = None, window: int = 0, chunk: int = 0,
-                 learned_sink: bool = False, projection_norm_eps: float | None = None) -> None:
+                 learned_sink: bool = False, projection_norm_eps: float | None = None, head_norm_eps: float | None = None,
+                 value_position: str | None = None, head_gate: bool = False) -> None:
         """Further options. `chunk` (instead of `window`): a position sees the keys of its own chunk of that many
         positions, chunks counted from position 0. `learned_sink`: exp(sink[h]), a learned number per head, in the
         softmax's denominator (instead of `sink`'s 1). `projection_norm_eps`: the whole q projection of a token (all
         heads at once), and likewise the whole k projection, is divided by its root mean square and multiplied by a
-        weight of that size (`q_norm`, `k_norm`, 32-bit) before the heads turn."""
+        weight of that size (`q_norm`, `k_norm`, 32-bit) before the heads turn. `head_norm_eps` (instead): every q head and
+        every k head is divided by its own root mean square and multiplied by a weight of the head's size that all heads
+        share (`q_norm`, `k_norm`), before the heads turn. `value_position` names a `rotary_frequencies` encoding over
+        all of `value_dim`: the value at position j is turned by j before it is cached, and each head's output at position
+        i is turned back by i. `head_gate`: each head's output (turned back) is multiplied by sigmoid(W_gate h)_head, one
+        number per head."""
+        if projection_norm_eps is not None and head_norm_eps is not None:
+            raise ValueError("a norm over the whole q and k projections or over every head, not both")
+        if head_gate and value_position is None:
+            raise ValueError("the gate per head rides on the kernel that turns the heads' outputs back (value_position)")
         if chunk < 0 or window < 0 or (chunk and window):
             raise ValueError("a sliding window or chunks (both >= 0), not both")
         if sink and learned_sink:
@@ -162,6 +172,8 @@ class GeneralAttention(Mixer):
         self.scale = scale if scale is not None else head_dim ** -0.5
         self.softcap, self.sink, self.qk_norm_eps, self.v_norm_eps, self.window = softcap, sink, qk_norm_eps, v_norm_eps, window
         self.chunk, self.learned_sink, self.projection_norm_eps = chunk, learned_sink, projection_norm_eps
+        self.head_norm_eps, self.value_position, self.head_gate = head_norm_eps, value_position, head_gate
+        self.gate: torch.Tensor | None = None
         self.qkv: torch.Tensor | None = None
         self.o: torch.Tensor | None = None
         self.q_norm: torch.Tensor | None = None
@@ -188,6 +200,11 @@ class GeneralAttention(Mixer):
         if self.projection_norm_eps is not None:
             specs["q_norm"] = ParamSpec((self.q_size,), "float32", init=(1.0, 0.1))
             specs["k_norm"] = ParamSpec((self.k_size,), "float32", init=(1.0, 0.1))
+        if self.head_norm_eps is not None:
+            specs["q_norm"] = ParamSpec((self.head_dim,), "float32", init=(1.0, 0.1))
+            specs["k_norm"] = ParamSpec((self.head_dim,), "float32", init=(1.0, 0.1))
+        if self.head_gate:
+            specs["gate"] = ParamSpec((self.num_heads, self.hidden_size))
         if self.learned_sink:
             specs["sinks"] = ParamSpec((self.num_heads,), "float32", init=(0.0, 1.0))
         return specs
@@ -208,12 +225,22 @@ class GeneralAttention(Mixer):
         qkv = linear(x, self.qkv, out_dtype=torch.float32, packed=self.qkv_packed)
         if self.projection_norm_eps is not None:         # in place, each over its whole stretch of the row
             hip.segment_rmsnorm_pair(qkv, (0, self.q_size, self.q_norm), (self.q_size, self.k_size, self.k_norm), self.projection_norm_eps)
+        value_enc = ctx.position_encodings[self.value_position] if self.value_position else None
+        if self.head_norm_eps is not None or value_enc is not None:      # in place: the heads' norms, the values' turn
+            hip.qkv_prepare(qkv, ctx.positions, self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim,
+                            q_weight=self.q_norm if self.head_norm_eps is not None else None,
+                            k_weight=self.k_norm if self.head_norm_eps is not None else None, eps=self.head_norm_eps or 0.0,
+                            value_freqs=None if value_enc is None else value_enc.frequencies(),
+                            value_interleaved=getattr(value_enc, "interleaved", False))
         q = hip.qkv_finish(qkv, enc.frequencies() if enc is not None else None, ctx.positions, slots, k_store, v_store,
                            self.num_heads, self.num_kv_heads, self.head_dim, self.value_dim, x.dtype,
                            interleaved=getattr(enc, "interleaved", True), qk_norm_eps=self.qk_norm_eps,
                            v_norm_eps=self.v_norm_eps, amplitude=getattr(enc, "amplitude", 1.0))
         o = hip.paged_attention(q, mem.k_cache, mem.v_cache, ctx, mem.space, self.scale, self.window, softcap=self.softcap,
                                 sink=self.sink, sinks=self.sinks, chunk_mask=self.chunk)
+        if value_enc is not None:                         # each head's sum turned back by its own position, then its gate
+            gate = linear(x, self.gate, out_dtype=torch.float32) if self.head_gate else None
+            hip.rotate_heads(o, o, value_enc.frequencies(), 1.0, ctx.positions, interleaved=value_enc.interleaved, back=True, gate=gate)
         return linear(o.view(ctx.num_tokens, self.num_heads * self.value_dim), self.o, out_dtype=torch.float32,
                       packed=self.o_packed)
 

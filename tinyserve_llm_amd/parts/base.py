@@ -197,11 +197,30 @@ class FeedForward(Part):
         raise NotImplementedError
 
 
+class TokenInput(Part):
+    """What a layer adds to the residual stream from the token ids themselves, beside its mixer and its feed-forward:
+    `forward(rows, ctx)` takes the stream's rows (in the engine's storage type) and gives 32-bit rows to be added,
+    through `post` if the part has one (a norm). A part that reads a second token table gets it from the embedding
+    (`attach`, called after `bind` with `Embedding.side_table()`)."""
+
+    post = None
+
+    def attach(self, table: torch.Tensor | None) -> None:
+        pass
+
+    def forward(self, rows: torch.Tensor, ctx: StepContext) -> torch.Tensor:
+        raise NotImplementedError
+
+
 class Embedding(Part):
     """Token ids to the first hidden rows [tokens, hidden]."""
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
+
+    def side_table(self) -> torch.Tensor | None:
+        """A second table [vocab, n] of per-token rows that layers read slices of (`TokenInput`), or None."""
+        return None
 
     def table(self) -> torch.Tensor | None:
         """The [vocab, hidden] matrix a tied head may share, or None if there is none to share."""
@@ -227,10 +246,12 @@ NORMS: dict[str, Callable[..., Norm]] = {}
 POSITION_ENCODINGS: dict[str, Callable[..., PositionEncoding]] = {}
 EMBEDDINGS: dict[str, Callable[..., Embedding]] = {}
 HEADS: dict[str, Callable[..., Head]] = {}
+TOKEN_INPUTS: dict[str, Callable[..., TokenInput]] = {}
 BLOCKS: dict[str, Callable[..., Any]] = {}
 
 _TABLES = {"mixer": MIXERS, "feed_forward": FEED_FORWARDS, "norm": NORMS,
-           "position_encoding": POSITION_ENCODINGS, "embedding": EMBEDDINGS, "head": HEADS, "block": BLOCKS}
+           "position_encoding": POSITION_ENCODINGS, "embedding": EMBEDDINGS, "head": HEADS, "block": BLOCKS,
+           "token_input": TOKEN_INPUTS}
 
 
 def register(family: str, name: str) -> Callable:

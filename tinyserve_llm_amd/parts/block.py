@@ -27,12 +27,13 @@ class Layer:
     norms: dict[str, Norm]           # by the names the arrangement uses
     block: str = "pre_norm"
     block_args: dict = field(default_factory=dict)      # the arrangement's own constants (a residual multiplier, say)
+    token_inputs: dict = field(default_factory=dict)    # parts that add something made from the token ids, by name
 
     def parts(self) -> dict[str, object]:
         """Every part by the name its parameters are known under (`layers.<i>.<name>.<parameter>`)."""
-        if {"mixer", "ff"} & set(self.norms):
-            raise ValueError("a norm cannot be named 'mixer' or 'ff'")
-        return {"mixer": self.mixer, "ff": self.feed_forward, **self.norms}
+        if {"mixer", "ff"} & (set(self.norms) | set(self.token_inputs)) or set(self.norms) & set(self.token_inputs):
+            raise ValueError("norms and token inputs have names of their own, other than 'mixer' and 'ff'")
+        return {"mixer": self.mixer, "ff": self.feed_forward, **self.norms, **self.token_inputs}
 
 
 def uses_norms(*names: str):
@@ -175,3 +176,29 @@ def pre_norm_stream_block(layer: Layer, hidden, residual, ctx: StepContext, mem:
         return stream, None
     x, h = stream.take(norms["norm2"])
     return ResidualStream(x, layer.feed_forward.forward(h, ctx)), None
+
+
+@register("block", "sandwich_scaled")
+@uses_norms("norm1", "norm1b", "scale1")
+@keeps_stream
+def sandwich_scaled_block(layer: Layer, hidden, residual, ctx: StepContext, mem: LayerMemory):
+    """x <- x + s1 * norm1b(mixer(norm1(x))), then x <- x + s2 * norm2b(feed_forward(norm2(x))) with RMS norms and learned
+    scales per channel ("scale1", "scale2": `parts.norm.ChannelScale`; "norm2", "norm2b", "scale2" only where the layer
+    has a feed-forward), then, for every token input of the layer in turn, x <- x + post(input(x, tokens)). The stream is
+    32-bit; each sum is left pending in it with the norm and the scale that the branch's rows still have to pass, so that
+    whoever takes the stream next does that norm, the sum and its own norm in one kernel."""
+    from tinyserve_llm_amd.parts.stream import ResidualStream
+    if not isinstance(hidden, ResidualStream) or residual is not None:
+        raise TypeError("this arrangement runs on a 32-bit residual stream (ModelSpec.residual_dtype = 'float32')")
+    norms = layer.norms
+    x, h = hidden.take(norms["norm1"])
+    stream = ResidualStream(x, layer.mixer.forward(h, ctx, mem), post=norms["norm1b"], scale=norms["scale1"].weight32)
+    if "norm2" in norms:
+        x, h = stream.take(norms["norm2"])
+        stream = ResidualStream(x, layer.feed_forward.forward(h, ctx), post=norms["norm2b"], scale=norms["scale2"].weight32)
+    elif layer.feed_forward.forward(None, ctx) is not None:
+        raise KeyError("a layer with a feed-forward names the norms 'norm2', 'norm2b' and 'scale2'")
+    for part in layer.token_inputs.values():
+        x, rows = stream.rows_as(part.operand_dtype)
+        stream = ResidualStream(x, part.forward(rows, ctx), post=part.post)
+    return stream, None

@@ -19,11 +19,15 @@ class TableEmbedding(Embedding):
     graph_safe = True
 
     def __init__(self, vocab_size: int, hidden_size: int, init: tuple[float, float] = (0.0, 0.02),
-                 float32_stream: bool = False, scale: float = 1.0, norm: "PartSpec | None" = None) -> None:
+                 float32_stream: bool = False, scale: float = 1.0, norm: "PartSpec | None" = None, side_width: int = 0,
+                 side_init: tuple[float, float] = (0.0, 1.0)) -> None:
         """`float32_stream`: the rows start a residual stream that is kept in 32-bit floats
         (`parts.stream.ResidualStream`) whatever the table's storage type; such rows may be multiplied
         by `scale` and passed through a norm that works element by element (`norm`: its PartSpec; its
-        parameters are the table's, named `norm_<name>`)."""
+        parameters are the table's, named `norm_<name>`). `side_width` > 0: a second table `side` [vocab, side_width] of
+        per-token rows that the layers' token inputs read stretches of (`parts.base.TokenInput`)."""
+        self.side_width, self.side_init = side_width, tuple(side_init)
+        self.side: torch.Tensor | None = None
         self.vocab_size, self.hidden_size, self.init = vocab_size, hidden_size, tuple(init)
         self.float32_stream, self.scale = float32_stream, scale
         if (scale != 1.0 or norm is not None) and not float32_stream:
@@ -35,6 +39,8 @@ class TableEmbedding(Embedding):
 
     def param_specs(self) -> dict[str, ParamSpec]:
         specs = {"weight": ParamSpec((self.vocab_size, self.hidden_size), init=self.init)}
+        if self.side_width:
+            specs["side"] = ParamSpec((self.vocab_size, self.side_width), init=self.side_init)
         if self.norm is not None:
             specs.update({f"norm_{name}": ps for name, ps in self.norm.param_specs().items()})
         return specs
@@ -46,6 +52,9 @@ class TableEmbedding(Embedding):
 
     def table(self) -> torch.Tensor | None:
         return self.weight
+
+    def side_table(self) -> torch.Tensor | None:
+        return self.side
 
     def forward(self, ctx: StepContext) -> "torch.Tensor | ResidualStream":
         if self.float32_stream and (self.scale != 1.0 or self.norm is not None):

@@ -91,12 +91,16 @@ class CappedGLU(FeedForward):
     """A gated feed-forward with capped branches: g = min(W_gate h, limit), u = clamp(W_up h, -limit, limit),
     W_down (g sigmoid(slope g) (u + up_shift)); limit <= 0: no cap. One fused projection gives gate | up as
     32-bit sums; the unit is taken in 32-bit and rounded to the storage type for the down projection, whose
-    result is 32-bit."""
+    result is 32-bit. `activation` "relu": the gate passes where it is positive, max(g, 0) (u + up_shift), instead of
+    through the sigmoid."""
 
     graph_safe = True
 
     def __init__(self, hidden_size: int, intermediate_size: int, limit: float = 0.0, slope: float = 1.702,
-                 up_shift: float = 1.0) -> None:
+                 up_shift: float = 1.0, activation: str = "sigmoid") -> None:
+        if activation not in ("sigmoid", "relu"):
+            raise ValueError(f"activation {activation!r}: 'sigmoid' (g sigmoid(slope g)) or 'relu'")
+        self.activation = activation
         self.hidden_size, self.intermediate_size = hidden_size, intermediate_size
         self.limit, self.slope, self.up_shift = limit, slope, up_shift
         self.gate_up: torch.Tensor | None = None
@@ -114,7 +118,7 @@ class CappedGLU(FeedForward):
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         sums = linear(x, self.gate_up, out_dtype=torch.float32, packed=self.gate_up_packed)
-        unit = hip.capped_glu(sums, self.limit, self.slope, self.up_shift, x.dtype)
+        unit = hip.capped_glu(sums, self.limit, self.slope, self.up_shift, x.dtype, relu=self.activation == "relu")
         return linear(unit, self.down, out_dtype=torch.float32, packed=self.down_packed)
 
 

@@ -20,14 +20,24 @@ class RoutedExperts(FeedForward):
     chosen (`correction` False: largest s); their weights are their s without the correction, over the chosen
     ones' sum (+ 1e-20) if `normalize`, times `router_scale`. `shared`: the constructor arguments of a
     `CappedGLU` that runs for every token and is added (None: no shared expert). The experts' matrices are
-    stacked: gate_up [experts, 2 ff, hidden], down [experts, hidden, ff]."""
+    stacked: gate_up [experts, 2 ff, hidden], down [experts, hidden, ff]. `scoring` "softmax_all": s is the softmax
+    over all the router's outputs instead of sigmoids. `identity`: the router has that many more outputs than there
+    are experts with matrices; they stand for experts that hand their input through (times the weight). `shared_gate`:
+    the shared expert's output is multiplied by sigmoid(w_sg . h), one number per token; w_sg is the router's last
+    row, so that its logit is 32-bit like the others."""
 
     graph_safe = True
 
     def __init__(self, hidden_size: int, num_experts: int, top: int, intermediate_size: int, limit: float = 0.0,
                  slope: float = 1.702, up_shift: float = 1.0, router_scale: float = 1.0, normalize: bool = True,
-                 correction: bool = True, shared: dict | None = None) -> None:
-        if not 1 <= top <= min(num_experts, hip.MOE_MAX_TOP) or num_experts > hip.MOE_MAX_EXPERTS:
+                 correction: bool = True, shared: dict | None = None, scoring: str = "sigmoid", identity: int = 0,
+                 shared_gate: bool = False) -> None:
+        if scoring not in ("sigmoid", "softmax_all") or identity < 0 or (shared_gate and shared is None):
+            raise ValueError("scoring 'sigmoid' or 'softmax_all'; identity >= 0; a gate on the shared expert needs one")
+        if top > num_experts + identity or num_experts + identity > hip.MOE_MAX_EXPERTS:
+            raise ValueError(f"top {top} of {num_experts} + {identity} experts, of which there may be {hip.MOE_MAX_EXPERTS}")
+        self.scoring, self.identity, self.shared_gate = scoring, identity, shared_gate
+        if not 1 <= top <= min(num_experts + identity, hip.MOE_MAX_TOP) or num_experts > hip.MOE_MAX_EXPERTS:
             raise ValueError(f"top {top} of {num_experts} experts: 1 <= top <= min(experts, {hip.MOE_MAX_TOP}), "
                              f"experts <= {hip.MOE_MAX_EXPERTS}")
         self.hidden_size, self.num_experts, self.top, self.intermediate_size = hidden_size, num_experts, top, intermediate_size
@@ -41,10 +51,10 @@ class RoutedExperts(FeedForward):
 
     def param_specs(self) -> dict[str, ParamSpec]:
         E, F, H = self.num_experts, self.intermediate_size, self.hidden_size
-        specs = {"router": ParamSpec((E, H), "float32", init=(0.0, 0.2)),
+        specs = {"router": ParamSpec((E + self.identity + int(self.shared_gate), H), "float32", init=(0.0, 0.2)),
                  "gate_up": ParamSpec((E, 2 * F, H)), "down": ParamSpec((E, H, F))}
         if self.has_correction:
-            specs["correction"] = ParamSpec((E,), "float32", init=(0.0, 0.1))
+            specs["correction"] = ParamSpec((E + self.identity,), "float32", init=(0.0, 0.1))
         if self.shared is not None:
             specs.update({f"shared_{name}": ps for name, ps in self.shared.param_specs().items()})
         return specs
@@ -63,13 +73,16 @@ class RoutedExperts(FeedForward):
         return self.shared.keep_streaming_copies() if self.shared is not None else 0
 
     def forward(self, x: torch.Tensor, ctx: StepContext) -> torch.Tensor:
-        experts, weights = hip.moe_route(x, self.router, self.correction, self.top, self.router_scale, self.normalize)
+        routed = hip.moe_route(x, self.router, self.correction, self.top, self.router_scale, self.normalize,
+                               softmax_all=self.scoring == "softmax_all", extras=int(self.shared_gate))
+        experts, weights = routed[0], routed[1]
         tile_rows = hip.moe_tile_rows(experts.numel(), self.num_experts, x.dtype, (self.hidden_size, self.intermediate_size))
         grouped = hip.moe_group(experts, self.num_experts, tile_rows)
         unit = hip.moe_gemm(x, self.gate_up, grouped, x.dtype, per_token=True, glu=(self.limit, self.slope, self.up_shift))
         rows = hip.moe_gemm(unit, self.down, grouped, torch.float32, per_token=False)
         shared = self.shared.forward(x, ctx) if self.shared is not None else None
-        return hip.moe_combine(rows, weights, shared)
+        return hip.moe_combine(rows, weights, shared, identity=(experts, self.num_experts, x) if self.identity else None,
+                               shared_gate=routed[2] if self.shared_gate else None)
 
 
 @register("feed_forward", "routed_dense_experts")

@@ -34,6 +34,7 @@ class RMSNorm(Norm):
     def bind(self, params) -> None:
         super().bind(params)
         self.applied = (1.0 + self.weight.float()).contiguous() if self.one_plus else self.weight
+        self.weight32 = self.applied if self.applied.dtype == torch.float32 else self.applied.float().contiguous()
 
     def __call__(self, x, residual=None, rows=None):
         if isinstance(x, ResidualStream):
@@ -56,6 +57,29 @@ class RMSNorm(Norm):
     def made_for(self, pending) -> bool:
         """Whether `pending` is this norm, deferred (by `defer` or through `request`)."""
         return isinstance(pending, DeferredNorm) and pending.weight is self.weight and pending.eps == self.eps
+
+
+@register("norm", "channel_scale")
+class ChannelScale(Norm):
+    """A learned factor per channel (a layer scale): x * weight, no statistics. In an arrangement that keeps a 32-bit
+    stream it rides on the kernel that adds a branch's rows (`ResidualStream(..., scale=weight32)`)."""
+
+    graph_safe = True
+
+    def __init__(self, hidden_size: int, init: float = 1.0) -> None:
+        self.hidden_size, self.init = hidden_size, init
+        self.weight: torch.Tensor | None = None
+        self.weight32: torch.Tensor | None = None
+
+    def param_specs(self) -> dict[str, ParamSpec]:
+        return {"weight": ParamSpec((self.hidden_size,), init=(self.init, 0.1))}
+
+    def bind(self, params) -> None:
+        super().bind(params)
+        self.weight32 = self.weight.float().contiguous()
+
+    def __call__(self, x, residual=None, rows=None):
+        raise TypeError("a channel scale is applied by the arrangement that names it, in the kernel that adds the branch")
 
 
 @register("norm", "dynamic_tanh")
