@@ -139,3 +139,42 @@ def bafarax_configs():
                                  window=130), D(640)),
         L("mlstm", M(heads=4, dim=64, vdim=128, gate_cap=12.0), D(640)), L("attention", s_att, E(experts=8, top=2, ff=128), weights_of=0)))
     return {"P": (P, 3), "Q": (Q, 4), "R": (R, 5), "S": (S, 6)}
+
+
+def tegolix_configs():
+    """Small Tegolix configurations that differ from each other in every size and option: the order of the two kinds of
+    mixer, key/value grouping, key and value head sizes (equal or not), how much of a head turns (all, part, none), a
+    frequency ramp or none, windows (one position, shorter and longer than a page, none), capped scores or not, the two
+    side scales, ranks of the decays' projections, recurrence heads from 4 to more than 256 dimensions, tau of 1, dense,
+    routed (no identity expert up to several, one choice up to all, with and without a shared expert) and absent
+    feed-forwards, a per-layer token input or none, and widths that are multiples of nothing."""
+    from tinyserve_llm_amd.config.bafarax import FrequencyRamp as Ramp, Rotation as Rot
+    from tinyserve_llm_amd.config.tegolix import TegolixConfig, TegolixDense as D, TegolixExperts as E, TegolixGLA as G, \
+        TegolixLayer as L, TegolixParallel as Par, TegolixRecurrence as R, TegolixWindowAttention as A
+    p_par = Par(A(heads=4, kv_heads=2, dim=32, vdim=48, scale=0.4, softcap=6.0, rot=Rot(16, 10000.0, Ramp(3.0, 64.0, 16.0, 2.0)), window=24),
+                R(heads=3, dim=20, decay_rank=8), left_scale=0.7, right_scale=1.2)
+    P = TegolixConfig(vocab=200, width=80, norm_eps=1e-6, side_dim=12, layers=(
+        L("gla", G(heads=3, dim=20, vdim=28, tau=8.0, decay_rank=8), D(96)),
+        L("parallel", p_par, E(experts=6, identity=2, top=3, ff=40, shared_ff=56)),
+        L("gla", G(heads=2, dim=16, vdim=40, tau=1.0, decay_rank=4), None)))
+    q_par = Par(A(heads=2, kv_heads=2, dim=16, vdim=16, scale=0.5, softcap=0.0, rot=Rot(16, 700.0), window=1),
+                R(heads=1, dim=16, decay_rank=16), left_scale=1.0, right_scale=1.0)
+    q_full = Par(A(heads=4, kv_heads=1, dim=8, vdim=24, scale=0.6, softcap=30.0, rot=Rot(0, 300.0), window=0),
+                 R(heads=2, dim=4, decay_rank=3), left_scale=1.5, right_scale=0.4)
+    Q = TegolixConfig(vocab=131, width=48, norm_eps=1e-4, side_dim=0, layers=(
+        L("parallel", q_par, E(experts=4, identity=0, top=1, ff=20, shared_ff=0)),
+        L("gla", G(heads=1, dim=16, vdim=16, tau=4.0, decay_rank=16), D(64)),
+        L("parallel", q_full, E(experts=3, identity=3, top=6, ff=12, shared_ff=24)),
+        L("gla", G(heads=1, dim=16, vdim=16, tau=4.0, decay_rank=16), None)))
+    # sizes that are multiples of nothing in particular: no kernel's fast path takes them
+    r_par = Par(A(heads=3, kv_heads=1, dim=20, vdim=12, scale=0.3, softcap=4.0, rot=Rot(10, 50000.0, Ramp(8.0, 32.0, 4.0, 1.0)), window=70),
+                R(heads=1, dim=300, decay_rank=5), left_scale=0.5, right_scale=2.0)
+    R_ = TegolixConfig(vocab=77, width=99, norm_eps=1e-5, side_dim=7, layers=(
+        L("parallel", r_par, D(52)), L("gla", G(heads=2, dim=18, vdim=270, tau=30.0, decay_rank=11), E(experts=5, identity=1, top=2, ff=17, shared_ff=0))))
+    # a width that the weight-streaming kernels take, heads of a matrix-core size, experts in tiles of several rows
+    s_par = Par(A(heads=8, kv_heads=2, dim=64, vdim=64, scale=0.2, softcap=15.0, rot=Rot(32, 250000.0), window=130),
+                R(heads=8, dim=64, decay_rank=32), left_scale=0.8, right_scale=0.9)
+    S = TegolixConfig(vocab=300, width=512, norm_eps=1e-6, side_dim=32, layers=(
+        L("gla", G(heads=4, dim=64, vdim=128, tau=16.0, decay_rank=16), E(experts=8, identity=2, top=2, ff=128, shared_ff=256)),
+        L("parallel", s_par, D(640)), L("gla", G(heads=8, dim=32, vdim=64, tau=12.0, decay_rank=16), D(640))))
+    return {"P": (P, 3), "Q": (Q, 4), "R": (R_, 5), "S": (S, 6)}

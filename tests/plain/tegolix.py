@@ -179,12 +179,24 @@ def chosen_experts(logits: torch.Tensor, correction: torch.Tensor, top: int) -> 
     return idx, torch.gather(s, 1, idx)
 
 
-def expert_mixture(h: torch.Tensor, W: dict, mlp: dict) -> torch.Tensor:
-    """The router's last `identity` outputs stand for experts that hand their input through."""
+def choice_margin(logits: torch.Tensor, correction: torch.Tensor, top: int) -> torch.Tensor:
+    """[n]: how far the last chosen expert's choice score lies above the best one left out (infinite where all are
+    chosen): a rounding of the scores by less than that chooses the same experts."""
+    ranked = torch.sort(torch.softmax(logits, dim=-1) + correction, dim=-1, descending=True).values
+    if top >= ranked.shape[-1]:
+        return torch.full(ranked.shape[:-1], float("inf"), dtype=ranked.dtype)
+    return ranked[..., top - 1] - ranked[..., top]
+
+
+def expert_mixture(h: torch.Tensor, W: dict, mlp: dict, margins: list | None = None) -> torch.Tensor:
+    """The router's last `identity` outputs stand for experts that hand their input through. `margins`, if given,
+    collects every token's `choice_margin`."""
     router = mlp["router"]
     real = int(router["experts"])
     silu = torch.nn.functional.silu
     idx, weights = chosen_experts(h @ W["router"].T, W["correction"], int(router["top"]))
+    if margins is not None:
+        margins.append(choice_margin(h @ W["router"].T, W["correction"], int(router["top"])))
     out = torch.zeros_like(h)
     for t in range(h.shape[0]):
         for w, e in zip(weights[t], idx[t]):
@@ -208,6 +220,7 @@ class PlainTegolix:
         self.memory: list[dict] = [dict() for _ in config["layers"]]
         self.fed = 0
         self.after_layers: list[torch.Tensor] = []      # the residual stream after every layer, of the last call
+        self.margins: torch.Tensor | None = None        # per token of the last call: the routers' smallest `choice_margin`
 
     @classmethod
     def from_folder(cls, folder: str, dtype: torch.dtype = torch.float64) -> "PlainTegolix":
@@ -231,6 +244,7 @@ class PlainTegolix:
         x = self.w["embed"][ids]
         side = int((c.get("token_side") or {}).get("dim", 0))
         self.after_layers = []
+        margins: list[torch.Tensor] = []
         for i, layer in enumerate(c["layers"]):
             p = f"l{i}."
             h = layer_norm(x, self.w[p + "norm1"], eps)
@@ -248,13 +262,14 @@ class PlainTegolix:
             if mlp is not None:
                 h = layer_norm(x, self.w[p + "norm2"], eps)
                 F = self._sub(p + "mlp.")
-                y = gated_unit(h, F, torch.relu) if mlp["kind"] == "dense" else expert_mixture(h, F, mlp)
+                y = gated_unit(h, F, torch.relu) if mlp["kind"] == "dense" else expert_mixture(h, F, mlp, margins)
                 x = x + layer_norm(y, self.w[p + "norm2b"], eps) * self.w[p + "ls2"]
             if side:
                 e = self.w["side.embed"][ids][:, i * side:(i + 1) * side]
                 y = (gelu_tanh(x @ self.w[p + "side.gate"].T) * e) @ self.w[p + "side.proj"].T
                 x = x + unit_rms(y, eps) * self.w[p + "side.norm"]
             self.after_layers.append(x.clone())
+        self.margins = torch.stack(margins).min(0).values if margins else torch.full((len(tokens),), float("inf"), dtype=x.dtype)
         return layer_norm(x, self.w["final.norm"], eps) @ self.w["head"].T
 
     def reset(self) -> None:
