@@ -38,6 +38,13 @@ output gate, and an mLSTM's matrix memory; dense and ungated routed feed-forward
 closest of the engine's models, at equal layer sizes and equal active parameters per token, in the same way. One JSON
 line.
 
+    python bench.py --tegolix [--shape 1b|3b] [--layers L] [--kernels-only]
+
+measures the Tegolix decoder (sandwiched RMS norms and learned scales per channel on a 32-bit stream, a per-layer token
+input, gated linear attention in turn with windowed attention beside a recurrence with token shift, dense and routed
+feed-forwards with identity experts and a gated shared expert) beside the Bafarax decoder, the closest of the engine's
+models, at equal layer sizes, in the same way. One JSON line.
+
     python bench.py --scenario requests-3b | chunked-8b [--layers L]
 
 runs a whole workload through `LLM.generate` instead and prints one JSON line of its own: many
@@ -854,6 +861,171 @@ def bafarax(args) -> int:
     return 0
 
 
+def tegolix_design(shape: str, layers: int | None):
+    """The Tegolix configuration that `--tegolix` measures at the layer sizes of `shape`, and those sizes by name."""
+    from tinyserve_llm_amd.config.bafarax import FrequencyRamp, Rotation
+    from tinyserve_llm_amd.config.tegolix import (TegolixConfig, TegolixDense, TegolixExperts, TegolixGLA, TegolixLayer, TegolixParallel,
+                                                  TegolixRecurrence, TegolixWindowAttention)
+    sizes = SHAPES[shape]
+    sh = sizes["shape"]
+    layers = layers or sizes["layers_full"]
+    hidden, nh, nkv, hd, inter, vocab = (sh["hidden_size"], sh["num_attention_heads"], sh["num_key_value_heads"], sh["head_dim"],
+                                         sh["intermediate_size"], sh["vocab_size"])
+    # gated linear attention of the matrix memory's sizes (8 heads, values twice as wide as keys); beside the windowed attention of
+    # the shape's heads a recurrence of heads of 64; 16 gated experts of an eighth of the dense width and two identity experts, of
+    # which a token uses 4, with a shared expert of half the dense width; 256 numbers of a second token table a layer
+    window, experts, identity, top, eff, sff, side = 1024, 16, 2, 4, inter // 8, inter // 2, 256
+    gh, gd, gv, rh, rd, rank = 8, hidden // 16, hidden // 8, hidden // 64, 64, 64
+    gla = TegolixGLA(heads=gh, dim=gd, vdim=gv, tau=16.0, decay_rank=rank)
+    left = TegolixWindowAttention(heads=nh, kv_heads=nkv, dim=hd, vdim=hd, scale=hd ** -0.5, softcap=30.0, window=window,
+                                  rot=Rotation(hd // 2, 10000.0, FrequencyRamp(factor=8.0, original=4096.0, fast=32.0, slow=1.0)))
+    par = TegolixParallel(left, TegolixRecurrence(heads=rh, dim=rd, decay_rank=rank), left_scale=0.6, right_scale=1.1)
+    moe, dense = TegolixExperts(experts=experts, identity=identity, top=top, ff=eff, shared_ff=sff), TegolixDense(inter)
+    cycle = (("gla", gla, dense), ("parallel", par, moe), ("gla", gla, dense), ("parallel", par, moe))
+    teg = TegolixConfig(vocab=vocab, width=hidden, norm_eps=1e-6, side_dim=side, layers=tuple(TegolixLayer(*cycle[i % 4]) for i in range(layers)))
+    return teg, dict(window=window, experts=experts, identity=identity, top=top, eff=eff, sff=sff, side=side, gh=gh, gd=gd, gv=gv, rh=rh, rd=rd, rank=rank)
+
+
+def tegolix(args) -> int:
+    """The Tegolix decoder beside the Bafarax decoder (the engine's closest design: a 32-bit stream with norms stored around
+    zero, a matrix memory, windowed attention, experts) at the layer sizes of `--shape`: whole-engine throughput, and the like
+    kernels of the two side by side. One JSON line."""
+    import torch
+
+    from tinyserve_llm_amd.ops import hip
+
+    baf, z = bafarax_design(args.shape, args.layers)
+    teg, t = tegolix_design(args.shape, args.layers)
+    layers, hidden, nh, nkv, hd, vocab = z["layers"], z["hidden"], z["nh"], z["nkv"], z["hd"], z["vocab"]
+    chunk, mh, md, mv = z["chunk"], z["mh"], z["md"], z["mv"]
+    window, gh, gd, gv, rh, rd = t["window"], t["gh"], t["gd"], t["gv"], t["rh"], t["rd"]
+    prompt_len = args.context
+    bench = DesignBench(vocab, prompt_len)
+    timed, context = bench.timed, bench.context
+    bf = torch.bfloat16
+
+    def kernel_pairs() -> dict:
+        pairs = {}
+        pool_page = 32
+        peaks = hip.measure_peaks()
+        read_peak, mfma_peak, vector_peak = peaks["read_GBps"] * 1e9, peaks["mfma_bf16_TFLOPs"] * 1e12, PEAK_FLOPS["fp32"]
+        sinks = torch.randn(nh, device="cuda")
+        for label, starts, counts in (("prompt portion", [0], [prompt_len]), ("decoded tokens, batch 64", [prompt_len + chunk // 2 - 1] * 64, [1] * 64)):
+            ctx, slots, pages = context(starts, counts, pool_page)
+            T, prompt, R = ctx.num_tokens, ctx.num_tokens > 64, len(starts)
+            of_peak = lambda flops, nbytes, us: ({"frac_of_mfma": flops / us * 1e6 / mfma_peak} if prompt else
+                                                 {"frac_of_read": nbytes / us * 1e6 / read_peak})
+            k = torch.randn(pages, nkv, pool_page, hd, device="cuda").to(bf).permute(0, 2, 1, 3)
+            v = torch.randn(pages, nkv, hd, pool_page, device="cuda").to(bf).permute(0, 3, 1, 2)
+            q = torch.randn(T, nh, hd, device="cuda").to(bf)
+            spans = list(zip(starts, counts))
+            seen_w = sum(min(p + 1, window) for s0, n in spans for p in range(s0, s0 + n))
+            seen_c = sum(p % chunk + 1 for s0, n in spans for p in range(s0, s0 + n))
+            # attention in a window with capped scores, against attention in chunks with learned sinks: the same kernels
+            us_t = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, window, softcap=30.0))
+            us_b = timed(lambda: hip.paged_attention(q, k, v, ctx, 0, hd ** -0.5, 0, sinks=sinks, chunk_mask=chunk))
+            pairs[f"attention, {label}"] = {
+                "tegolix_us": us_t, "bafarax_us": us_b, "tegolix_keys": seen_w, "bafarax_keys": seen_c,
+                "tegolix": of_peak(4 * nh * hd * seen_w, seen_w * 2 * nkv * hd * 2, us_t),
+                "bafarax": of_peak(4 * nh * hd * seen_c, seen_c * 2 * nkv * hd * 2, us_b)}
+            # between projection and cache: the heads' weighted norms, the values' turn, the rotation and the cache write, and after
+            # attention the turn back with the gate per head; against the norms over the whole q and k and the rotation
+            qkv_row = (nh + 2 * nkv) * hd
+            qkv32 = torch.randn(T, qkv_row, device="cuda")
+            nw, qw, kw = torch.ones(hd, device="cuda"), torch.ones(nh * hd, device="cuda"), torch.ones(nkv * hd, device="cuda")
+            rfreqs = torch.rand(hd // 2, dtype=torch.float64, device="cuda")
+            hfreqs = torch.rand(hd // 4, dtype=torch.float64, device="cuda")
+            gate = torch.randn(T, nh, device="cuda")
+            o16 = torch.randn(T, nh, hd, device="cuda").to(bf)
+
+            def teg_finish():
+                hip.qkv_prepare(qkv32, ctx.positions, nh, nkv, hd, hd, q_weight=nw, k_weight=nw, eps=1e-6, value_freqs=rfreqs)
+                out = hip.qkv_finish(qkv32, hfreqs, ctx.positions, slots, k, v, nh, nkv, hd, hd, bf, interleaved=False, amplitude=1.2)
+                hip.rotate_heads(o16, o16, rfreqs, 1.0, ctx.positions, interleaved=False, back=True, gate=gate)
+                return out
+
+            def baf_finish():
+                hip.segment_rmsnorm_pair(qkv32, (0, nh * hd, qw), (nh * hd, nkv * hd, kw), 1e-6)
+                return hip.qkv_finish(qkv32, rfreqs, ctx.positions, slots, k, v, nh, nkv, hd, hd, bf, interleaved=False)
+            us_t, us_b = timed(teg_finish), timed(baf_finish)
+            tbytes, bbytes = T * (qkv_row * (4 + 4 + 4 + 2) + nh * hd * 4), T * qkv_row * (4 + 4 + 4 + 2)
+            pairs[f"between projection and cache, {label}"] = {
+                "tegolix_us": us_t, "bafarax_us": us_b, "tegolix_bytes": tbytes, "bafarax_bytes": bbytes,
+                "tegolix_frac_of_read": tbytes / us_t * 1e6 / read_peak, "bafarax_frac_of_read": bbytes / us_b * 1e6 / read_peak}
+            # the stream's sum and the norm that reads it: with the branch's own norm and scale on the way in, against the sum alone
+            x32, a32 = torch.randn(T, hidden, device="cuda"), torch.randn(T, hidden, device="cuda")
+            w32 = torch.ones(hidden, device="cuda")
+            us_t = timed(lambda: hip.stream_post_norm(x32, a32, w32, w32, 1e-6, w32, 1e-6, bf))
+            us_b = timed(lambda: hip.stream_update_norm(x32, a32, None, None, 1.0, (w32, None), 1e-6, out_dtype=bf))
+            sbytes = T * hidden * (3 * 4 + 2)
+            pairs[f"stream sum and norm, {label}"] = {"tegolix_us": us_t, "bafarax_us": us_b, "bytes": sbytes,
+                                                      "tegolix_frac_of_read": sbytes / us_t * 1e6 / read_peak,
+                                                      "bafarax_frac_of_read": sbytes / us_b * 1e6 / read_peak}
+            # the recurrences: gated linear attention (scan, then the heads' norm and gate) and the recurrence with token shift,
+            # against the matrix memory at the gated linear attention's sizes
+            gproj = torch.randn(T, 2 * gh * gd + 2 * gh * gv, device="cuda")
+            gz, gbias, gnorm = torch.randn(T, gh * gd, device="cuda"), torch.full((gh * gd,), 3.0, device="cuda"), torch.ones(gv, device="cuda")
+            gstate = torch.zeros(R, gh * gd * gv, device="cuda")
+            K, V = gh * gd, gh * gv
+
+            def gla():
+                o = hip.decay_scan(gproj[:, :K], gproj[:, K:2 * K], gproj[:, 2 * K:2 * K + V], gz, gbias, gstate, ctx.cu_seqlens, ctx.state_slots,
+                                   gh, gd, gv, form="sigmoid_root", tau=16.0, q_scale=gd ** -0.5)
+                return hip.mlstm_finish(o, gnorm, gproj[:, 2 * K + V:], gh, gv, 1e-6, bf, silu_gate=True)
+            us_gla = timed(gla)
+            us_gla_scan = timed(lambda: hip.decay_scan(gproj[:, :K], gproj[:, K:2 * K], gproj[:, 2 * K:2 * K + V], gz, gbias, gstate, ctx.cu_seqlens,
+                                                       ctx.state_slots, gh, gd, gv, form="sigmoid_root", tau=16.0, q_scale=gd ** -0.5))
+            rr, rk, rv, rg, rz = (torch.randn(T, rh * rd, device="cuda") for _ in range(5))
+            rbias, rbonus, rnorm = torch.full((rh * rd,), -3.0, device="cuda"), torch.randn(rh, rd, device="cuda"), torch.ones(rh * rd, device="cuda")
+            rstate = torch.zeros(R, rh * rd * rd + hidden, device="cuda")
+            h16, mu = torch.randn(T, hidden, device="cuda").to(bf), torch.rand(5, hidden, device="cuda")
+
+            def shifted():
+                kept = rstate[:, rh * rd * rd:]
+                mixes = hip.token_shift(h16, mu, kept, ctx)
+                hip.token_shift_keep(kept, h16, ctx)
+                o = hip.decay_scan(rr, rk, rv, rz, rbias, rstate, ctx.cu_seqlens, ctx.state_slots, rh, rd, rd, form="double_exponent", bonus=rbonus)
+                return mixes, hip.mlstm_finish(o, rnorm, rg, rh, rd, 1e-6, bf, silu_gate=True)
+            us_shift = timed(shifted)
+            width = 2 * mh * md + mh * mv + 2 * mh + mh * mv
+            proj = torch.randn(T, width, device="cuda")
+            gb = torch.zeros(2 * mh, device="cuda")
+            mstate = torch.zeros(R, hip.mlstm_state_size(mh, md, mv), device="cuda")
+            mw = torch.ones(mh * mv, device="cuda")
+
+            def memory():
+                o = hip.mlstm_scan(proj, gb[:mh], gb[mh:], mstate, ctx.cu_seqlens, ctx.state_slots, mh, md, mv, 15.0,
+                                   host_cu_seqlens=ctx.host_cu_seqlens, scratch=ctx.scratch)
+                return hip.mlstm_finish(o, mw, proj[:, width - mh * mv:], mh, mv, 1e-6, bf)
+            us_b = timed(memory)
+            gbytes = T * (3 * K + 2 * V) * 4 + T * V * (4 + 4 + 2) + 2 * R * gstate.shape[1] * 4
+            sbytes = T * (5 * rh * rd * 4 + hidden * 2 * 6 + rh * rd * (4 + 4 + 2)) + 2 * R * rstate.shape[1] * 4
+            mbytes = T * width * 4 + T * mh * mv * (4 + 4 + 2) + 2 * R * mstate.shape[1] * 4
+            gflops, sflops, mflops = 4 * T * gh * gd * gv, 4 * T * rh * rd * rd, 4 * T * mh * md * mv
+            pairs[f"recurrence, {label}"] = {
+                "tegolix_gla_us": us_gla, "tegolix_gla_scan_us": us_gla_scan, "tegolix_shifted_us": us_shift, "bafarax_memory_us": us_b,
+                "tegolix_gla_bytes": gbytes, "tegolix_shifted_bytes": sbytes, "bafarax_memory_bytes": mbytes, "tegolix_gla_flops_fp32": gflops,
+                "tegolix_shifted_flops_fp32": sflops, "bafarax_memory_flops_fp32": mflops,
+                "tegolix_gla_frac_of_read": gbytes / us_gla * 1e6 / read_peak, "tegolix_shifted_frac_of_read": sbytes / us_shift * 1e6 / read_peak,
+                "bafarax_memory_frac_of_read": mbytes / us_b * 1e6 / read_peak,
+                "tegolix_gla_frac_of_fp32_vector": gflops / us_gla * 1e6 / vector_peak,
+                "tegolix_shifted_frac_of_fp32_vector": sflops / us_shift * 1e6 / vector_peak,
+                "bafarax_memory_frac_of_fp32_vector": mflops / us_b * 1e6 / vector_peak}
+        pairs["peaks"] = {"read_GBps": read_peak / 1e9, "mfma_bf16_TFLOPs": mfma_peak / 1e12, "fp32_vector_TFLOPs_published": vector_peak / 1e12}
+        return pairs
+
+    record = {"designs": {} if args.kernels_only else {"bafarax": bench.whole_engine(baf), "tegolix": bench.whole_engine(teg)},
+              "kernels": kernel_pairs(),
+              "config": {"shape": args.shape, "layers": layers, "hidden": hidden, "heads": nh, "kv_heads": nkv, "head_dim": hd,
+                         "tegolix": {k: v for k, v in t.items()},
+                         "tegolix_layers": "in turn: gated linear attention with a dense feed-forward, windowed attention beside a recurrence "
+                                           "with token shift, with experts",
+                         "bafarax_memory": {"heads": mh, "dim": md, "vdim": mv}, "bafarax_chunk": chunk,
+                         "vocab": vocab, "context": prompt_len, "dtype": "bf16", "data": "synthetic uniform token ids, random weights"}}
+    print(json.dumps(record))
+    return 0
+
+
 def kernel_classes(llm, config, batch: int, reps: int = 5) -> dict:
     """Times one decode step's kernels by class. An eager step (no graph) is run once with every
     launch of the engine's kernel module noted down with its operands; then each class's launches
@@ -987,7 +1159,9 @@ def main() -> int:
     ap.add_argument("--bafarax", action="store_true",
                     help="measure the Bafarax decoder beside the Fanotar decoder at the layer sizes of --shape: whole-engine "
                          "throughput and the like kernels side by side; one JSON line")
-    ap.add_argument("--kernels-only", action="store_true", help="with --bafarax: the kernels side by side, no whole-engine runs")
+    ap.add_argument("--tegolix", action="store_true",
+                    help="the Tegolix decoder beside the Bafarax decoder at the layer sizes of --shape: throughput and like kernels")
+    ap.add_argument("--kernels-only", action="store_true", help="with --bafarax or --tegolix: the kernels side by side, no whole-engine runs")
     ap.add_argument("--kernel-classes", action="store_true",
                     help="time one decode step's kernels class by class (bytes, microseconds, GB/s) and exit")
     ap.add_argument("--peaks", action="store_true",
@@ -1017,6 +1191,8 @@ def main() -> int:
         return fanotar(args)
     if args.bafarax:
         return bafarax(args)
+    if args.tegolix:
+        return tegolix(args)
     sizes = SHAPES[args.shape]
     full_layers = sizes["layers_full"]
     args.layers = args.layers or full_layers
