@@ -970,11 +970,11 @@ def tegolix(args) -> int:
 
             def gla():
                 o = hip.decay_scan(gproj[:, :K], gproj[:, K:2 * K], gproj[:, 2 * K:2 * K + V], gz, gbias, gstate, ctx.cu_seqlens, ctx.state_slots,
-                                   gh, gd, gv, form="sigmoid_root", tau=16.0, q_scale=gd ** -0.5)
+                                   gh, gd, gv, form="sigmoid_root", tau=16.0, q_scale=gd ** -0.5, longest=max(counts))
                 return hip.mlstm_finish(o, gnorm, gproj[:, 2 * K + V:], gh, gv, 1e-6, bf, silu_gate=True)
             us_gla = timed(gla)
             us_gla_scan = timed(lambda: hip.decay_scan(gproj[:, :K], gproj[:, K:2 * K], gproj[:, 2 * K:2 * K + V], gz, gbias, gstate, ctx.cu_seqlens,
-                                                       ctx.state_slots, gh, gd, gv, form="sigmoid_root", tau=16.0, q_scale=gd ** -0.5))
+                                                       ctx.state_slots, gh, gd, gv, form="sigmoid_root", tau=16.0, q_scale=gd ** -0.5, longest=max(counts)))
             rr, rk, rv, rg, rz = (torch.randn(T, rh * rd, device="cuda") for _ in range(5))
             rbias, rbonus, rnorm = torch.full((rh * rd,), -3.0, device="cuda"), torch.randn(rh, rd, device="cuda"), torch.ones(rh * rd, device="cuda")
             rstate = torch.zeros(R, rh * rd * rd + hidden, device="cuda")
@@ -984,7 +984,7 @@ def tegolix(args) -> int:
                 kept = rstate[:, rh * rd * rd:]
                 mixes = hip.token_shift(h16, mu, kept, ctx)
                 hip.token_shift_keep(kept, h16, ctx)
-                o = hip.decay_scan(rr, rk, rv, rz, rbias, rstate, ctx.cu_seqlens, ctx.state_slots, rh, rd, rd, form="double_exponent", bonus=rbonus)
+                o = hip.decay_scan(rr, rk, rv, rz, rbias, rstate, ctx.cu_seqlens, ctx.state_slots, rh, rd, rd, form="double_exponent", bonus=rbonus, longest=max(counts))
                 return mixes, hip.mlstm_finish(o, rnorm, rg, rh, rd, 1e-6, bf, silu_gate=True)
             us_shift = timed(shifted)
             width = 2 * mh * md + mh * mv + 2 * mh + mh * mv

@@ -117,7 +117,7 @@ def scan_case(read_first: bool, H: int, D: int, V: int, counts_by_step, slots, t
         K = H * D
         o = h.decay_scan(fused[:, :K], fused[:, K:2 * K], fused[:, 2 * K:], cat(z), bias.to(DEV), state, dev(cu), dev([slots[r] for r in live]),
                          H, D, V, form="double_exponent" if read_first else "sigmoid_root", tau=tau, q_scale=1.0 if read_first else D ** -0.5,
-                         bonus=None if bonus is None else bonus.to(DEV))
+                         bonus=None if bonus is None else bonus.to(DEV), longest=max(step))
         for i, r in enumerate(live):
             got[r].append(o[cu[i]:cu[i + 1]].cpu())
             fed[r] += step[r]
@@ -179,6 +179,26 @@ def test_the_bonus_is_for_the_current_token_only_and_tau_roots_the_decay():
     h.decay_scan(one(1.0), one(1.0), one(8.0), one(0.0), torch.zeros(1, device=DEV), state, **args, form="sigmoid_root", tau=2.0)
     o = h.decay_scan(one(1.0), one(0.0), one(0.0), one(0.0), torch.zeros(1, device=DEV), state, **args, form="sigmoid_root", tau=2.0)
     assert float(o) == pytest.approx(8.0 * math.sqrt(0.5), rel=1e-6), "sigmoid(0)^(1/2), applied before the read-out"
+
+
+@pytest.mark.parametrize("read_first", [False, True])
+@pytest.mark.parametrize("sizes", [(2, 64, 128), (3, 20, 64), (1, 256, 256), (2, 128, 72)])
+def test_wide_and_narrow_slices_of_the_columns_give_the_same_bits(read_first, sizes):
+    """Steps of few tokens a request give a wave 64 value columns, steps of many 16: a request decoded token by token and the
+    same request fed whole must not differ by a bit."""
+    h = hip()
+    H, D, V = sizes
+    gen = torch.Generator().manual_seed(D)
+    n = 9
+    q, k, z = (torch.randn(n, H * D, generator=gen).to(DEV) for _ in range(3))
+    v = torch.randn(n, H * V, generator=gen).to(DEV)
+    bias, bonus = torch.randn(H * D, generator=gen).to(DEV), torch.randn(H, D, generator=gen).to(DEV)
+    kw = dict(heads=H, dim=D, vdim=V, form="double_exponent" if read_first else "sigmoid_root", tau=2.0, bonus=bonus if read_first else None)
+    whole_state, stepped_state = torch.zeros(1, H * D * V, device=DEV), torch.zeros(1, H * D * V, device=DEV)
+    whole = h.decay_scan(q, k, v, z, bias, whole_state, dev([0, n]), dev([0]), **kw, longest=n)
+    stepped = torch.cat([h.decay_scan(q[t:t + 1], k[t:t + 1], v[t:t + 1], z[t:t + 1], bias, stepped_state, dev([0, 1]), dev([0]), **kw, longest=1)
+                         for t in range(n)])
+    assert torch.equal(whole, stepped) and torch.equal(whole_state, stepped_state)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

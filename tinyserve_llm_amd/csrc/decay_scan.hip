@@ -2,16 +2,18 @@
 // at a request's start. For a token with q, k [dim], v [vdim] and decays w [dim] in (0, 1) there are two orders:
 //     decay first  (gated linear attention):   S' = diag(w) S + k v^T,  o = S'^T q;
 //     read first   (RWKV-style, with a bonus): o = (S + diag(u) k v^T)^T q,  S' = diag(w) S + k v^T,
-// u [heads, dim] a learned bonus that only the current token's k v^T gets. The decays come from raw sums z and a bias
-// b per head and channel, in 32-bit:
-//     sigmoid form:      w = sigmoid(z + b)^(1 / tau) = exp(logsigmoid(z + b) / tau);
-//     double exponent:   w = exp(-exp(z + b)).
+// u [heads, dim] a learned bonus that only the current token's k v^T gets.
+//   * `ts_decay_factors`: the decays from raw sums z and a bias b per head and channel, in 32-bit:
+//     sigmoid form w = sigmoid(z + b)^(1 / tau) = exp(logsigmoid(z + b) / tau); double exponent w = exp(-exp(z + b)).
 //   * `ts_decay_scan`: one workgroup per (request, head, slice of the value columns) walks the request's tokens of
-//     the step in order. A wave owns 16 (or 4) value columns; a lane keeps a share of the rows of one column of S in
-//     registers, the lanes that share a column add their parts up through the wave's own exchanges, so a token
-//     needs no barrier: only a block of tokens does, whose q, k, w and v go through LDS together (the next block's
-//     loads are in flight while this one is worked on). The state is read from the request's slot at the start and
-//     written back at the end. A column's sum runs over the rows in an order that the sizes alone fix.
+//     the step in order. A wave owns 16 value columns (four lanes share a column's rows and add their parts up
+//     through the wave's own exchanges) or 64 (a lane keeps a whole column, in four partial sums that it adds in the
+//     exchanges' order: the same result bit for bit), so a token needs no barrier: only a block of tokens does, whose
+//     q, k, w and v go through LDS together, in 16-byte pieces whose places a thread works out once; the next block's
+//     loads are in flight while this one is worked on. The state is read from the request's slot at the start and
+//     written back at the end. A column's sum runs over the rows in an order that the sizes alone fix. Heads of more
+//     than 256 dimensions, and sizes or places that are no whole 16-byte pieces, take a kernel that fetches element
+//     by element, with 4 columns a wave.
 //   * `ts_token_shift`: x_s[t] = h[t] + (h[t-1] - h[t]) mu_s for several mixes s at once, h[t-1] of a request's first
 //     token of the step being the row its state slot keeps (zeros for a new request); `ts_token_shift_keep` then
 //     leaves each request's last row of the step in its slot.
@@ -29,10 +31,10 @@ static __device__ __forceinline__ float ds_decay(float z, int form, float inv_ta
 template <int WC, int R4, bool READ_FIRST>
 __global__ void __launch_bounds__(256)
 decay_scan_kernel(float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
-                  int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ z,
-                  int64_t z_stride, const float* __restrict__ z_bias, const float* __restrict__ bonus,
+                  int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ w,
+                  int64_t w_stride, const float* __restrict__ bonus,
                   float* __restrict__ state, int64_t state_stride, const int32_t* __restrict__ cu_seqlens,
-                  const int32_t* __restrict__ state_slots, int heads, int dim, int vdim, int form, float inv_tau,
+                  const int32_t* __restrict__ state_slots, int heads, int dim, int vdim,
                   float q_scale, int block_tokens) {
   extern __shared__ float lds[];
   constexpr int GROUPS = TS_WAVE / WC;
@@ -65,7 +67,7 @@ decay_scan_kernel(float* __restrict__ out, const float* __restrict__ q, int64_t 
     if (p < 2 * dim4) return p - dim4 < dim ? k[t * k_stride + h * dim + p - dim4] : 0.f;
     if (p < 3 * dim4) {
       const int d = p - 2 * dim4;
-      return d < dim ? ds_decay(z[t * z_stride + h * dim + d] + z_bias[h * dim + d], form, inv_tau) : 1.f;
+      return d < dim ? w[t * w_stride + h * dim + d] : 1.f;
     }
     const int c = p - 3 * dim4;
     return v0 + c < vdim ? v[t * v_stride + h * vdim + v0 + c] : 0.f;
@@ -135,6 +137,180 @@ decay_scan_kernel(float* __restrict__ out, const float* __restrict__ q, int64_t 
     }
 }
 
+// The same walk where everything comes in whole 16-byte pieces (dim and vdim multiples of four up to 256 dimensions,
+// rows and places 16-byte aligned). A column's rows are dealt out in fours to GROUPS shares (4 for heads of less than 128
+// dimensions, else 16): share g takes the fours g, g + GROUPS, ... in ascending order, and the shares' sums meet in a
+// tree (neighbours first). Narrow form: a share is a lane, 64 / GROUPS columns a wave, the tree is the wave's exchanges.
+// Wide form (steps of few tokens a request): a lane keeps a whole column and all its shares' sums, 64 columns a wave, so
+// that the state's rows are read and written whole cache lines at a time; the tree is the same, so is every bit of the
+// result. RG: fours of rows a share takes. A thread carries up to NP pieces of every token of a block of TB tokens: which
+// ones, from where and to where it works out once.
+template <int GROUPS, bool WIDE, int RG, bool READ_FIRST, int NP, int TB>
+__global__ void __launch_bounds__(256)
+decay_scan_pieces_kernel(float* __restrict__ out, const float* __restrict__ q, int64_t q_stride, const float* __restrict__ k,
+                         int64_t k_stride, const float* __restrict__ v, int64_t v_stride, const float* __restrict__ w,
+                         int64_t w_stride, const float* __restrict__ bonus, float* __restrict__ state, int64_t state_stride,
+                         const int32_t* __restrict__ cu_seqlens, const int32_t* __restrict__ state_slots, int heads, int dim,
+                         int vdim, float q_scale) {
+  extern __shared__ float lds[];
+  constexpr int WC = WIDE ? TS_WAVE : TS_WAVE / GROUPS;     // columns of a wave
+  constexpr int VG = WIDE ? GROUPS : 1;                     // shares of a column that a lane keeps
+  // per token in LDS: q | k | w, each padded with zeros to the rows that the shares walk (so that no read of a row has to
+  // ask whether the row exists: a branch there would keep a token's reads from going out together), then the slice's v;
+  // behind the two blocks of tokens, the bonus (padded likewise) where there is one
+  constexpr int DIMP = RG * GROUPS * 4;
+  const int threads = blockDim.x, waves = threads / TS_WAVE;
+  const int cols = waves * WC;
+  const int in_size = 3 * DIMP + cols;
+  const int seq = blockIdx.x, h = blockIdx.y, v0 = blockIdx.z * cols;
+  const int wave = threadIdx.x / TS_WAVE, lane = threadIdx.x & (TS_WAVE - 1);
+  const int col = wave * WC + (lane % WC), grp = WIDE ? 0 : lane / WC;
+  const bool live = v0 + col < vdim;
+  const int t_begin = cu_seqlens[seq], t_end = cu_seqlens[seq + 1];
+  if (t_begin >= t_end) return;
+  float* st = state + (int64_t)state_slots[seq] * state_stride + (int64_t)h * dim * vdim;
+  float S[RG * VG * 4];
+#pragma unroll
+  for (int r = 0; r < RG; ++r)
+#pragma unroll
+    for (int g = 0; g < VG; ++g)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = (r * GROUPS + grp + g) * 4 + j;
+        S[(r * VG + g) * 4 + j] = (live && d < dim) ? st[(int64_t)d * vdim + v0 + col] : 0.f;
+      }
+  // this thread's pieces of a token: source (at token 0), stride from token to token, place in the token's row of LDS
+  const int d4 = dim / 4, pieces = 3 * d4 + cols / 4;
+  const float* src[NP];
+  int64_t stride[NP];
+  float mult[NP];
+  bool has[NP];
+  int place[NP];
+#pragma unroll
+  for (int i = 0; i < NP; ++i) {
+    const int p = threadIdx.x + i * threads;
+    has[i] = p < pieces;
+    mult[i] = 1.f;
+    src[i] = q;
+    stride[i] = 0;
+    place[i] = 0;
+    if (p < d4) { src[i] = q + h * dim + 4 * p; stride[i] = q_stride; mult[i] = q_scale; place[i] = 4 * p; }
+    else if (p < 2 * d4) { src[i] = k + h * dim + 4 * (p - d4); stride[i] = k_stride; place[i] = DIMP + 4 * (p - d4); }
+    else if (p < 3 * d4) { src[i] = w + h * dim + 4 * (p - 2 * d4); stride[i] = w_stride; place[i] = 2 * DIMP + 4 * (p - 2 * d4); }
+    else if (p < pieces) {
+      const int c = 4 * (p - 3 * d4);
+      has[i] = v0 + c < vdim;                               // (a slice's last columns may lie beyond the head: zeros)
+      src[i] = v + h * vdim + v0 + c;
+      stride[i] = v_stride;
+      place[i] = 3 * DIMP + c;
+    }
+  }
+  float4 staged[NP][TB];
+  auto load = [&](int t0, int nt) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i)
+#pragma unroll
+      for (int tl = 0; tl < TB; ++tl) {
+        float4 x = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (has[i] && tl < nt) x = *(const float4*)(src[i] + (int64_t)(t0 + tl) * stride[i]);
+        staged[i][tl] = make_float4(x.x * mult[i], x.y * mult[i], x.z * mult[i], x.w * mult[i]);
+      }
+  };
+  auto store = [&](float* dst) {
+#pragma unroll
+    for (int i = 0; i < NP; ++i) {
+      const int p = threadIdx.x + i * threads;
+      if (p < pieces) {
+#pragma unroll
+        for (int tl = 0; tl < TB; ++tl) *(float4*)(dst + tl * in_size + place[i]) = staged[i][tl];
+      }
+    }
+  };
+  const int block_size = TB * in_size;
+  float* u_s = lds + 2 * block_size;
+  if (DIMP != dim)
+    for (int e = threadIdx.x; e < 2 * block_size; e += threads) lds[e] = 0.f;      // (the pads, once: no store goes there again)
+  if constexpr (READ_FIRST)
+    for (int e = threadIdx.x; e < DIMP; e += threads) u_s[e] = e < dim ? bonus[h * dim + e] : 0.f;
+  load(t_begin, min(TB, t_end - t_begin));
+  if (DIMP != dim) __syncthreads();
+  store(lds);
+  __syncthreads();
+  int buf = 0;
+  for (int t0 = t_begin; t0 < t_end; t0 += TB, buf ^= 1) {
+    const int nt = min(TB, t_end - t0);
+    const int next_n = min(TB, t_end - t0 - TB);
+    if (next_n > 0) load(t0 + TB, next_n);
+    const float* base = lds + buf * block_size;
+    auto token = [&](int tl) {
+      const float* q_s = base + tl * in_size;
+      const float* k_s = q_s + DIMP;
+      const float* w_s = k_s + DIMP;
+      const float vc = w_s[DIMP + col];
+      float o[VG];
+#pragma unroll
+      for (int g = 0; g < VG; ++g) o[g] = 0.f;
+#pragma unroll
+      for (int r = 0; r < RG; ++r)
+#pragma unroll
+        for (int g = 0; g < VG; ++g) {
+          const int d0 = (r * GROUPS + grp + g) * 4;         // (a row beyond the head: k = 0 keeps its S at 0, q = 0 adds nothing)
+          const float4 q4 = *(const float4*)(q_s + d0), k4 = *(const float4*)(k_s + d0), w4 = *(const float4*)(w_s + d0);
+          const float qq[4] = {q4.x, q4.y, q4.z, q4.w}, kk[4] = {k4.x, k4.y, k4.z, k4.w}, ww[4] = {w4.x, w4.y, w4.z, w4.w};
+          float uu[4] = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (READ_FIRST) {
+            const float4 u4 = *(const float4*)(u_s + d0);
+            uu[0] = u4.x; uu[1] = u4.y; uu[2] = u4.z; uu[3] = u4.w;
+          }
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const float kv = kk[j] * vc;
+            float& s = S[(r * VG + g) * 4 + j];
+            if constexpr (READ_FIRST) {
+              o[g] = fmaf(fmaf(uu[j], kv, s), qq[j], o[g]);
+              s = fmaf(ww[j], s, kv);
+            } else {
+              s = fmaf(ww[j], s, kv);
+              o[g] = fmaf(s, qq[j], o[g]);
+            }
+          }
+        }
+      float sum;
+      if constexpr (!WIDE) {
+        sum = o[0];
+#pragma unroll
+        for (int off = WC; off < TS_WAVE; off <<= 1) sum += __shfl_xor(sum, off, TS_WAVE);
+      } else {
+#pragma unroll
+        for (int span = 1; span < VG; span <<= 1)
+#pragma unroll
+          for (int g = 0; g < VG; g += 2 * span) o[g] += o[g + span];
+        sum = o[0];
+      }
+      if (grp == 0 && live) out[(int64_t)(t0 + tl) * heads * vdim + h * vdim + v0 + col] = sum;
+    };
+    if (!WIDE && nt == TB) {
+      // a whole block: its tokens side by side in the code, so that a token's reads of LDS and the exchange of the one
+      // before it go on behind the other's arithmetic (the state is the only thing one token hands the next)
+#pragma unroll
+      for (int tl = 0; tl < TB; ++tl) token(tl);
+    } else {
+      for (int tl = 0; tl < nt; ++tl) token(tl);
+    }
+    if (next_n > 0) store(lds + (buf ^ 1) * block_size);
+    __syncthreads();
+  }
+#pragma unroll
+  for (int r = 0; r < RG; ++r)
+#pragma unroll
+    for (int g = 0; g < VG; ++g)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int d = (r * GROUPS + grp + g) * 4 + j;
+        if (live && d < dim) st[(int64_t)d * vdim + v0 + col] = S[(r * VG + g) * 4 + j];
+      }
+}
+
 // Tokens of a block for a workgroup of `threads`: as many as a thread can carry and 64 KB of LDS hold twice.
 static int ds_block_tokens(int threads, int in_size) {
   int n = (DS_MAX_STAGED * threads) / in_size;
@@ -144,15 +320,55 @@ static int ds_block_tokens(int threads, int in_size) {
   return n;
 }
 
+// `wide`: a wave owns 64 columns instead of 16 (steps of few tokens a request: the state's rows are read and written
+// whole cache lines at a time, and nothing is exchanged between lanes); the result is the same bit for bit.
 extern "C" int ts_decay_scan(float* out, const float* q, int64_t q_stride, const float* k, int64_t k_stride, const float* v,
-                             int64_t v_stride, const float* z, int64_t z_stride, const float* z_bias, const float* bonus,
-                             float* state, int64_t state_stride, const int32_t* cu_seqlens, const int32_t* state_slots,
-                             int num_seqs, int heads, int dim, int vdim, int form, float tau, float q_scale, int read_first,
-                             int waves, hipStream_t stream) {
+                             int64_t v_stride, const float* w, int64_t w_stride, const float* bonus, float* state,
+                             int64_t state_stride, const int32_t* cu_seqlens, const int32_t* state_slots, int num_seqs, int heads,
+                             int dim, int vdim, float q_scale, int read_first, int waves, int wide, hipStream_t stream) {
   if (num_seqs <= 0) return TS_OK;
-  if (heads <= 0 || heads > 65535 || dim <= 0 || dim > 1024 || vdim <= 0 || waves < 1 || waves > 4 || (form != 0 && form != 1) ||
-      !(tau > 0.f) || (read_first && !bonus) || state_stride < (int64_t)heads * dim * vdim)
+  if (heads <= 0 || heads > 65535 || dim <= 0 || dim > 1024 || vdim <= 0 || waves < 1 || waves > 4 || (read_first && !bonus) ||
+      state_stride < (int64_t)heads * dim * vdim)
     return TS_BAD_SHAPE;
+  const bool pieces = dim <= 256 && dim % 4 == 0 && vdim % 4 == 0 && ((q_stride | k_stride | v_stride | w_stride | state_stride) & 3) == 0 &&
+                      (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)w) & 15) == 0;
+  if (pieces) {
+    const int groups = dim < 128 ? 4 : 16;                  // (by the head's size alone: both forms then sum in one order)
+    if (!wide && groups == 16) waves = 4;                   // (4 columns a wave: a workgroup's waves share what is staged)
+    const int wc = wide ? 64 : TS_WAVE / groups;
+    const int cols = waves * wc;
+    const int slices = (vdim + cols - 1) / cols;
+    if (slices > 65535) return TS_BAD_SHAPE;
+    const int threads = waves * TS_WAVE;
+    const int np = ((3 * dim + cols) / 4 + threads - 1) / threads;
+    const int fours = (dim / 4 + groups - 1) / groups;      // fours of rows a share takes,
+    const int rg = fours <= 1 ? 1 : fours <= 2 ? 2 : fours <= 4 ? 4 : 8;      // as the instances have them
+    const int in_size = 3 * rg * groups * 4 + cols;
+    dim3 grid(num_seqs, heads, slices);
+#define DS_FARGS out, q, q_stride, k, k_stride, v, v_stride, w, w_stride, bonus, state, state_stride, cu_seqlens, state_slots, heads, dim, \
+                 vdim, q_scale
+#define DS_FAST3(G, WD, RG, RF, NP, TB) \
+    decay_scan_pieces_kernel<G, WD, RG, RF, NP, TB><<<grid, threads, (size_t)(2 * TB * in_size + rg * groups * 4) * sizeof(float), stream>>>(DS_FARGS)
+#define DS_FAST2(G, WD, RG, NP, TB) \
+    { if (np > NP) return TS_BAD_SHAPE; if (read_first) { DS_FAST3(G, WD, RG, true, NP, TB); } else { DS_FAST3(G, WD, RG, false, NP, TB); } }
+    // (pieces of a token that a thread carries, by the head's size whatever the workgroup's waves; at most 16 pieces in
+    // flight, a block of at most 8 tokens)
+    if (groups == 4) {
+#define DS_FAST1(WD) \
+      if (rg == 1) DS_FAST2(4, WD, 1, 1, 8) else if (rg == 2) DS_FAST2(4, WD, 2, 1, 8) else if (rg == 4) DS_FAST2(4, WD, 4, 1, 8) \
+      else DS_FAST2(4, WD, 8, 2, 8)
+      if (wide) { DS_FAST1(true) } else { DS_FAST1(false) }
+#undef DS_FAST1
+    } else if (wide) {
+      if (rg <= 2) DS_FAST2(16, true, 2, 2, 8) else DS_FAST2(16, true, 4, 4, 4)
+    } else {
+      if (rg <= 2) DS_FAST2(16, false, 2, 1, 8) else DS_FAST2(16, false, 4, 1, 8)
+    }
+#undef DS_FAST2
+#undef DS_FAST3
+#undef DS_FARGS
+    return ts_check_launch();
+  }
   const int wc = dim <= 256 ? 16 : 4;                       // longer heads: more lanes share a column
   const int groups = TS_WAVE / wc;
   if (wc == 4) waves = 4;                                   // (their rows of q, k and w need a whole workgroup's hands)
@@ -166,8 +382,8 @@ extern "C" int ts_decay_scan(float* out, const float* q, int64_t q_stride, const
   const int r4 = (dim4 / 4 + groups - 1) / groups;          // fours of rows a lane keeps
   dim3 grid(num_seqs, heads, slices);
   const size_t lds = (size_t)2 * block_tokens * in_size * sizeof(float);
-#define DS_ARGS out, q, q_stride, k, k_stride, v, v_stride, z, z_stride, z_bias, bonus, state, state_stride, cu_seqlens, state_slots, \
-                heads, dim, vdim, form, 1.0f / tau, q_scale, block_tokens
+#define DS_ARGS out, q, q_stride, k, k_stride, v, v_stride, w, w_stride, bonus, state, state_stride, cu_seqlens, state_slots, \
+                heads, dim, vdim, q_scale, block_tokens
 #define DS_LAUNCH(WC, R4) \
   if (read_first) decay_scan_kernel<WC, R4, true><<<grid, waves * TS_WAVE, lds, stream>>>(DS_ARGS); \
   else decay_scan_kernel<WC, R4, false><<<grid, waves * TS_WAVE, lds, stream>>>(DS_ARGS)
@@ -185,6 +401,28 @@ extern "C" int ts_decay_scan(float* out, const float* q, int64_t q_stride, const
   }
 #undef DS_LAUNCH
 #undef DS_ARGS
+  return ts_check_launch();
+}
+
+// w = sigmoid(z + b)^(1 / tau) (form 0) or exp(-exp(z + b)) (form 1), element by element; b repeats every `width`.
+__global__ void __launch_bounds__(256)
+decay_factors_kernel(float* __restrict__ w, const float* __restrict__ z, int64_t z_stride, const float* __restrict__ bias, int width,
+                     int64_t total, int form, float inv_tau) {
+  for (int64_t at = (int64_t)blockIdx.x * 256 + threadIdx.x; at < total; at += (int64_t)gridDim.x * 256) {
+    const int64_t t = at / width;
+    const int i = (int)(at - t * width);
+    w[at] = ds_decay(z[t * z_stride + i] + bias[i], form, inv_tau);
+  }
+}
+
+extern "C" int ts_decay_factors(float* w, const float* z, int64_t z_stride, const float* bias, int num_tokens, int width, int form,
+                                float tau, hipStream_t stream) {
+  if (num_tokens <= 0) return TS_OK;
+  if (width <= 0 || z_stride < width || (form != 0 && form != 1) || !(tau > 0.f)) return TS_BAD_SHAPE;
+  const int64_t total = (int64_t)num_tokens * width;
+  int64_t blocks = (total + 255) / 256;
+  if (blocks > 16384) blocks = 16384;
+  decay_factors_kernel<<<(unsigned)blocks, 256, 0, stream>>>(w, z, z_stride, bias, width, total, form, 1.0f / tau);
   return ts_check_launch();
 }
 

@@ -281,11 +281,71 @@ stream_post_norm_kernel(float* __restrict__ x, const float* __restrict__ a, cons
     rs_store(h, h_code, r * width + i, w ? xr[i] * inv * w[i] : xr[i]);
 }
 
+// The same for rows of up to RS_THREADS * HELD elements: every load of the row, the branch and the weights goes out before
+// the first is used, and the row stays in registers between the sums of squares and the scalings (a lane beyond the row
+// reads the row's last element and stores nothing). The sums are taken by the same tree over the same lanes' parts.
+template <typename H, int HELD>
+__global__ void __launch_bounds__(RS_THREADS)
+stream_post_norm_held_kernel(float* __restrict__ x, const float* __restrict__ a, const float* __restrict__ post_w,
+                             const float* __restrict__ scale, float post_eps, H* __restrict__ h, const float* __restrict__ w,
+                             float eps, int width) {
+  __shared__ float scratch[RS_THREADS / TS_WAVE];
+  const int64_t r = blockIdx.x;
+  float* xr = x + r * width;
+  const float* ar = a + r * width;
+  const float* sc = scale ? scale : post_w;
+  const float* wn = w ? w : post_w;
+  float v[HELD], va[HELD], pw[HELD], ps[HELD], nw[HELD];
+#pragma unroll
+  for (int j = 0; j < HELD; ++j) {
+    const int i = min(threadIdx.x + j * RS_THREADS, width - 1);
+    v[j] = xr[i];
+    va[j] = ar[i];
+    pw[j] = post_w[i];
+    ps[j] = sc[i];
+    nw[j] = wn[i];
+  }
+  float squares = 0.f;
+#pragma unroll
+  for (int j = 0; j < HELD; ++j) squares = threadIdx.x + j * RS_THREADS < width ? fmaf(va[j], va[j], squares) : squares;
+  const float inv_a = 1.0f / sqrtf(block_sum(squares, scratch) / (float)width + post_eps);
+  squares = 0.f;
+#pragma unroll
+  for (int j = 0; j < HELD; ++j) {
+    const int i = threadIdx.x + j * RS_THREADS;
+    float add = va[j] * inv_a * pw[j];
+    if (scale) add *= ps[j];
+    v[j] += add;
+    if (i < width) {
+      xr[i] = v[j];
+      squares = fmaf(v[j], v[j], squares);
+    }
+  }
+  if (!h) return;
+  float inv = 1.0f;
+  if (w) inv = 1.0f / sqrtf(block_sum(squares, scratch) / (float)width + eps);
+#pragma unroll
+  for (int j = 0; j < HELD; ++j) {
+    const int i = threadIdx.x + j * RS_THREADS;
+    if (i < width) Num<H>::st(h + r * width + i, w ? v[j] * inv * nw[j] : v[j]);
+  }
+}
+
 extern "C" int ts_stream_post_norm(float* x, const float* a, const float* post_w, const float* scale, float post_eps, void* h,
                                    int h_dtype, const float* w, float eps, int num_rows, int width, hipStream_t stream) {
   if (num_rows <= 0) return TS_OK;
   if (width <= 0 || !x || !a || !post_w) return TS_BAD_SHAPE;
   if (h_dtype != 0 && h_dtype != 1) return TS_BAD_DTYPE;
+  if (width <= RS_THREADS * RS_HELD) {
+#define RS_POST(H, HELD) \
+    stream_post_norm_held_kernel<H, HELD><<<num_rows, RS_THREADS, 0, stream>>>(x, a, post_w, scale, post_eps, (H*)h, w, eps, width)
+#define RS_POST_H(H) \
+    if (width <= RS_THREADS * 4) { RS_POST(H, 4); } else if (width <= RS_THREADS * 8) { RS_POST(H, 8); } else { RS_POST(H, RS_HELD); }
+    if (h_dtype == 0) { RS_POST_H(float) } else { RS_POST_H(bf16_t) }
+#undef RS_POST_H
+#undef RS_POST
+    return ts_check_launch();
+  }
   stream_post_norm_kernel<<<num_rows, RS_THREADS, 0, stream>>>(x, a, post_w, scale, post_eps, h, h_dtype, w, eps, width);
   return ts_check_launch();
 }

@@ -109,7 +109,8 @@ def _declare(lib: ctypes.CDLL) -> None:
         "ts_mlstm_scan_chunks": [p, p, i64, p, p, p, p, p, p, p, p, p, i, i, i, i, i, f, f, p],
         "ts_mlstm_finish": [p, i, p, p, p, i64, i, i, i, f, i, i, p],
         "ts_moe_combine": [p, p, p, p, i, i, i, p, i, p, i, p, p],
-        "ts_decay_scan": [p, p, i64, p, i64, p, i64, p, i64, p, p, p, i64, p, p, i, i, i, i, i, f, f, i, i, p],
+        "ts_decay_scan": [p, p, i64, p, i64, p, i64, p, i64, p, p, i64, p, p, i, i, i, i, f, i, i, i, p],
+        "ts_decay_factors": [p, p, i64, p, i, i, i, f, p],
         "ts_token_shift": [p, p, i, p, p, i64, p, p, p, i, i, i, p],
         "ts_token_shift_keep": [p, i64, p, i, p, p, i, i, p],
         "ts_stream_post_norm": [p, p, p, p, f, p, i, p, f, i, i, p],
@@ -2424,17 +2425,20 @@ def mlstm_finish(o: torch.Tensor, weight: torch.Tensor, gate: torch.Tensor, head
 DECAY_FORMS = {"sigmoid_root": 0, "double_exponent": 1}
 DECAY_MAX_DIM = 1024
 DECAY_FULL_WORKGROUPS = 512      # workgroups of four waves from which a step keeps them (fewer: one wave each, four times as many)
+DECAY_WIDE_UP_TO = 4             # tokens of a step's longest portion up to which a wave owns 64 value columns instead of 16
 
 
 def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, z_bias: torch.Tensor, state: torch.Tensor,
                cu_seqlens: torch.Tensor, state_slots: torch.Tensor, heads: int, dim: int, vdim: int, *, form: str, tau: float = 1.0,
-               q_scale: float = 1.0, bonus: torch.Tensor | None = None) -> torch.Tensor:
+               q_scale: float = 1.0, bonus: torch.Tensor | None = None, longest: int | None = None) -> torch.Tensor:
     """Linear attention with a decay per key channel over a packed step. q, k, z float32 [tokens, heads dim] and v
     float32 [tokens, heads vdim] are views whose rows may lie apart (columns of fused projections); z_bias float32
     [heads dim]. The decays are w = sigmoid(z + z_bias)^(1 / tau) (`form` "sigmoid_root") or exp(-exp(z + z_bias))
     ("double_exponent"). Without `bonus`: S <- diag(w) S + k v^T, o = S^T (q q_scale). With `bonus` (float32 [heads, dim]):
     o = (S + diag(bonus) k v^T)^T q first, then the same update. `state` float32 [slots, >= heads dim vdim]: each
-    request's S lies at the start of its slot's row, is read there and written back. Returns o float32 [tokens, heads vdim]."""
+    request's S lies at the start of its slot's row, is read there and written back. Returns o float32 [tokens, heads vdim].
+    `longest`: the most tokens any request feeds in the step (None: unknown); steps of few tokens a request are cut into
+    fewer, wider slices of the value columns (the result is the same bit for bit)."""
     _gpu(q, k, v, z, z_bias, state, cu_seqlens, state_slots, bonus)
     T = q.shape[0]
     _need(form in DECAY_FORMS, lambda: f"form {form!r}: one of {sorted(DECAY_FORMS)}")
@@ -2449,11 +2453,17 @@ def decay_scan(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tenso
     _need(cu_seqlens.dtype == torch.int32 and cu_seqlens.shape == (S + 1,) and state_slots.dtype == torch.int32, "cu_seqlens int32 [requests + 1], slots int32 [requests]")
     _need(0 < dim <= DECAY_MAX_DIM and tau > 0, lambda: f"heads of up to {DECAY_MAX_DIM} dimensions, a positive tau")
     out = torch.empty((T, heads * vdim), dtype=torch.float32, device=q.device)
-    waves = 4 if vdim >= 64 and S * heads * (vdim // 64) >= DECAY_FULL_WORKGROUPS else 1
+    w = torch.empty((T, heads * dim), dtype=torch.float32, device=q.device)
+    _run("decay_factors", library().ts_decay_factors(_ptr(w), _ptr(z), z.stride(0), _ptr(z_bias), T, heads * dim, DECAY_FORMS[form], float(tau), _stream()))
+    wide = longest is not None and longest <= DECAY_WIDE_UP_TO and vdim >= 64
+    if wide:
+        waves = min(4, vdim // 64)
+    else:
+        waves = 4 if vdim >= 64 and S * heads * (vdim // 64) >= DECAY_FULL_WORKGROUPS else 1
     _run("decay_scan", library().ts_decay_scan(
-        _ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(z), z.stride(0), _ptr(z_bias), _ptr(bonus),
-        _ptr(state), state.stride(0), _ptr(cu_seqlens), _ptr(state_slots), S, heads, dim, vdim, DECAY_FORMS[form], float(tau),
-        float(q_scale), int(bonus is not None), waves, _stream()))
+        _ptr(out), _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _ptr(w), w.stride(0), _ptr(bonus),
+        _ptr(state), state.stride(0), _ptr(cu_seqlens), _ptr(state_slots), S, heads, dim, vdim, float(q_scale), int(bonus is not None),
+        waves, int(wide), _stream()))
     return out
 
 

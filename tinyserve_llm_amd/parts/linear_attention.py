@@ -69,7 +69,7 @@ class GatedLinearAttention(Mixer):
         z = linear(linear(x, self.decay_down), self.decay_up, out_dtype=torch.float32)
         o = hip.decay_scan(proj[:, :K], proj[:, K:2 * K], proj[:, 2 * K:2 * K + V], z, self.decay_bias, mem.state, ctx.cu_seqlens,
                            ctx.state_slots, H, self.head_dim, self.value_dim, form="sigmoid_root", tau=self.tau,
-                           q_scale=float(self.head_dim) ** -0.5)
+                           q_scale=float(self.head_dim) ** -0.5, longest=ctx.max_query_len)
         gated = hip.mlstm_finish(o, self.norm, proj[:, 2 * K + V:], H, self.value_dim, self.norm_eps, x.dtype, silu_gate=True)
         return linear(gated, self.o, out_dtype=torch.float32, packed=self.o_packed)
 
@@ -128,6 +128,6 @@ class ShiftedDecayRecurrence(Mixer):
         low = linear(mixes[4], self.decay_down, out_dtype=torch.float32)
         z = linear(hip.bias_activation(low, None, "tanh", x.dtype), self.decay_up, out_dtype=torch.float32)
         o = hip.decay_scan(r, k, v, z, self.decay_bias, mem.state, ctx.cu_seqlens, ctx.state_slots, H, D, D,
-                           form="double_exponent", bonus=self.bonus)
+                           form="double_exponent", bonus=self.bonus, longest=ctx.max_query_len)
         gated = hip.mlstm_finish(o, self.norm, g, H, D, self.norm_eps, x.dtype, silu_gate=True)
         return linear(gated, self.o, out_dtype=torch.float32, packed=self.packed.get("o"))
