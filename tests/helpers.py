@@ -177,4 +177,13 @@ def tegolix_configs():
     S = TegolixConfig(vocab=300, width=512, norm_eps=1e-6, side_dim=32, layers=(
         L("gla", G(heads=4, dim=64, vdim=128, tau=16.0, decay_rank=16), E(experts=8, identity=2, top=2, ff=128, shared_ff=256)),
         L("parallel", s_par, D(640)), L("gla", G(heads=8, dim=32, vdim=64, tau=12.0, decay_rank=16), D(640))))
-    return {"P": (P, 3), "Q": (Q, 4), "R": (R_, 5), "S": (S, 6)}
+    # two pairs of mixers with windows of their own (one longer than most prompts, one shorter than a page), heads of the
+    # matrix-core kernels' sizes with and without a cap, a pair first and without a feed-forward, more identity experts than others
+    t_wide = Par(A(heads=8, kv_heads=4, dim=128, vdim=128, scale=0.09, softcap=0.0, rot=Rot(128, 500000.0), window=300),
+                 R(heads=4, dim=64, decay_rank=8), left_scale=1.3, right_scale=0.7)
+    t_short = Par(A(heads=4, kv_heads=1, dim=96, vdim=96, scale=0.1, softcap=10.0, rot=Rot(32, 20000.0, Ramp(4.0, 128.0, 16.0, 1.0)), window=50),
+                  R(heads=8, dim=32, decay_rank=24), left_scale=0.5, right_scale=1.0)
+    T = TegolixConfig(vocab=160, width=256, norm_eps=1e-5, side_dim=20, layers=(
+        L("parallel", t_wide, None), L("gla", G(heads=4, dim=32, vdim=32, tau=9.0, decay_rank=12), E(experts=2, identity=5, top=1, ff=48, shared_ff=64)),
+        L("parallel", t_short, D(320)), L("gla", G(heads=2, dim=128, vdim=64, tau=20.0, decay_rank=6), D(192))))
+    return {"P": (P, 3), "Q": (Q, 4), "R": (R_, 5), "S": (S, 6), "T": (T, 7)}

@@ -402,7 +402,7 @@ def test_relu_gated_unit():
 
 # ---- whole models through trace replay ---------------------------------------------------------------
 
-LENGTHS = {"P": [1, 23, 97, 200], "Q": [1, 30, 75, 150], "R": [2, 19, 66, 131], "S": [1, 40, 140]}
+LENGTHS = {"P": [1, 23, 97, 200], "Q": [1, 30, 75, 150], "R": [2, 19, 66, 131], "S": [1, 40, 140], "T": [3, 50, 120]}
 TOL = {"float32": 2e-4, "bfloat16": 6e-2}       # of the spread of the oracle's logits
 # A router's choice is discrete: where the oracle's last chosen expert leads the best one left out by less than the
 # engine's rounding of the scores, either choice is right, and what follows in the request (the states carry it on) is
@@ -428,7 +428,7 @@ class Rows:
         return self.logits[pos]
 
 
-@pytest.fixture(scope="module", params=["P", "Q", "R", "S"])
+@pytest.fixture(scope="module", params=["P", "Q", "R", "S", "T"])
 def case(request, tmp_path_factory):
     from tinyserve_llm_amd.weights.random_init import write_random_model
     name = request.param

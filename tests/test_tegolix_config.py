@@ -25,7 +25,7 @@ from tinyserve_llm_amd.weights.random_init import write_random_model
 F64 = torch.float64
 
 
-@pytest.mark.parametrize("name", ["P", "Q", "R", "S"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T"])
 def test_configuration_round_trip_and_folder(name, tmp_path):
     config, seed = tegolix_configs()[name]
     raw = config.to_dict()

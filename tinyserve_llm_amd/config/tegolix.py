@@ -20,12 +20,12 @@ class TegolixGLA:
     dim: int
     vdim: int
     tau: float
-    decay_rank: int = 16         # inner size of the decays' two projections (the checkpoint's `a1` has that many rows)
+    decay_rank: int = 32         # inner size of the decays' two projections (the checkpoint's `a1` has that many rows)
 
     @classmethod
     def from_dict(cls, raw: Mapping[str, Any], where: str) -> "TegolixGLA":
         c = cls(heads=int(_need(raw, "heads", where)), dim=int(_need(raw, "dim", where)), vdim=int(_need(raw, "vdim", where)),
-                tau=float(_need(raw, "tau", where)), decay_rank=int(raw.get("decay_rank", 16)))
+                tau=float(_need(raw, "tau", where)), decay_rank=int(raw.get("decay_rank", 32)))
         if min(c.heads, c.dim, c.vdim, c.decay_rank) <= 0 or not c.tau > 0:
             raise ConfigError(f"{where}: heads, dim, vdim and tau are positive")
         return c
@@ -73,11 +73,11 @@ class TegolixWindowAttention:
 class TegolixRecurrence:
     heads: int
     dim: int
-    decay_rank: int = 16         # (the checkpoint's `w1` has that many rows)
+    decay_rank: int = 32         # (the checkpoint's `w1` has that many rows)
 
     @classmethod
     def from_dict(cls, raw: Mapping[str, Any], where: str) -> "TegolixRecurrence":
-        c = cls(heads=int(_need(raw, "heads", where)), dim=int(_need(raw, "dim", where)), decay_rank=int(raw.get("decay_rank", 16)))
+        c = cls(heads=int(_need(raw, "heads", where)), dim=int(_need(raw, "dim", where)), decay_rank=int(raw.get("decay_rank", 32)))
         if min(c.heads, c.dim, c.decay_rank) <= 0:
             raise ConfigError(f"{where}: heads and dim are positive")
         return c
