@@ -138,7 +138,7 @@ decay_scan_kernel(float* __restrict__ out, const float* __restrict__ q, int64_t 
 }
 
 // The same walk where everything comes in whole 16-byte pieces (dim and vdim multiples of four up to 256 dimensions,
-// rows and places 16-byte aligned). A column's rows are dealt out in fours to GROUPS shares (4 for heads of less than 128
+// rows and places 16-byte aligned). A column's rows are dealt out in fours to GROUPS shares (4 for heads of less than 64
 // dimensions, else 16): share g takes the fours g, g + GROUPS, ... in ascending order, and the shares' sums meet in a
 // tree (neighbours first). Narrow form: a share is a lane, 64 / GROUPS columns a wave, the tree is the wave's exchanges.
 // Wide form (steps of few tokens a request): a lane keeps a whole column and all its shares' sums, 64 columns a wave, so
@@ -242,7 +242,7 @@ decay_scan_pieces_kernel(float* __restrict__ out, const float* __restrict__ q, i
     const int next_n = min(TB, t_end - t0 - TB);
     if (next_n > 0) load(t0 + TB, next_n);
     const float* base = lds + buf * block_size;
-    auto token = [&](int tl) {
+    auto token = [&](int tl) -> float {
       const float* q_s = base + tl * in_size;
       const float* k_s = q_s + DIMP;
       const float* w_s = k_s + DIMP;
@@ -275,27 +275,39 @@ decay_scan_pieces_kernel(float* __restrict__ out, const float* __restrict__ q, i
             }
           }
         }
-      float sum;
-      if constexpr (!WIDE) {
-        sum = o[0];
-#pragma unroll
-        for (int off = WC; off < TS_WAVE; off <<= 1) sum += __shfl_xor(sum, off, TS_WAVE);
-      } else {
+      if constexpr (WIDE) {                                  // the shares' sums, neighbours first
 #pragma unroll
         for (int span = 1; span < VG; span <<= 1)
 #pragma unroll
           for (int g = 0; g < VG; g += 2 * span) o[g] += o[g + span];
-        sum = o[0];
       }
+      return o[0];
+    };
+    auto put = [&](int tl, float sum) {
       if (grp == 0 && live) out[(int64_t)(t0 + tl) * heads * vdim + h * vdim + v0 + col] = sum;
     };
     if (!WIDE && nt == TB) {
-      // a whole block: its tokens side by side in the code, so that a token's reads of LDS and the exchange of the one
-      // before it go on behind the other's arithmetic (the state is the only thing one token hands the next)
+      // a whole block: its tokens side by side in the code (the state is the only thing one token hands the next), and the
+      // lanes' shares of all its tokens meet afterwards, stage by stage for the eight tokens at once: an exchange waits a
+      // hundred cycles for its answer, and a token's four in a row were most of what a token cost
+      float part[TB];
 #pragma unroll
-      for (int tl = 0; tl < TB; ++tl) token(tl);
+      for (int tl = 0; tl < TB; ++tl) part[tl] = token(tl);
+#pragma unroll
+      for (int off = WC; off < TS_WAVE; off <<= 1)
+#pragma unroll
+        for (int tl = 0; tl < TB; ++tl) part[tl] += __shfl_xor(part[tl], off, TS_WAVE);
+#pragma unroll
+      for (int tl = 0; tl < TB; ++tl) put(tl, part[tl]);
     } else {
-      for (int tl = 0; tl < nt; ++tl) token(tl);
+      for (int tl = 0; tl < nt; ++tl) {
+        float sum = token(tl);
+        if constexpr (!WIDE) {
+#pragma unroll
+          for (int off = WC; off < TS_WAVE; off <<= 1) sum += __shfl_xor(sum, off, TS_WAVE);
+        }
+        put(tl, sum);
+      }
     }
     if (next_n > 0) store(lds + (buf ^ 1) * block_size);
     __syncthreads();
@@ -333,7 +345,7 @@ extern "C" int ts_decay_scan(float* out, const float* q, int64_t q_stride, const
   const bool pieces = dim <= 256 && dim % 4 == 0 && vdim % 4 == 0 && ((q_stride | k_stride | v_stride | w_stride | state_stride) & 3) == 0 &&
                       (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)w) & 15) == 0;
   if (pieces) {
-    const int groups = dim < 128 ? 4 : 16;                  // (by the head's size alone: both forms then sum in one order)
+    const int groups = dim < 64 ? 4 : 16;                   // (by the head's size alone: both forms then sum in one order)
     if (!wide && groups == 16) waves = 4;                   // (4 columns a wave: a workgroup's waves share what is staged)
     const int wc = wide ? 64 : TS_WAVE / groups;
     const int cols = waves * wc;
@@ -352,17 +364,18 @@ extern "C" int ts_decay_scan(float* out, const float* q, int64_t q_stride, const
 #define DS_FAST2(G, WD, RG, NP, TB) \
     { if (np > NP) return TS_BAD_SHAPE; if (read_first) { DS_FAST3(G, WD, RG, true, NP, TB); } else { DS_FAST3(G, WD, RG, false, NP, TB); } }
     // (pieces of a token that a thread carries, by the head's size whatever the workgroup's waves; at most 16 pieces in
-    // flight, a block of at most 8 tokens)
+    // flight. The narrow form takes blocks of 16 tokens where LDS holds two of them: a block's loads have the time the
+    // block before takes to be worked on, and that has to cover a trip to memory)
     if (groups == 4) {
-#define DS_FAST1(WD) \
-      if (rg == 1) DS_FAST2(4, WD, 1, 1, 8) else if (rg == 2) DS_FAST2(4, WD, 2, 1, 8) else if (rg == 4) DS_FAST2(4, WD, 4, 1, 8) \
-      else DS_FAST2(4, WD, 8, 2, 8)
-      if (wide) { DS_FAST1(true) } else { DS_FAST1(false) }
-#undef DS_FAST1
+      if (wide) {
+        if (rg == 1) DS_FAST2(4, true, 1, 1, 8) else if (rg == 2) DS_FAST2(4, true, 2, 1, 8) else DS_FAST2(4, true, 4, 1, 8)
+      } else {
+        if (rg == 1) DS_FAST2(4, false, 1, 1, 16) else if (rg == 2) DS_FAST2(4, false, 2, 1, 16) else DS_FAST2(4, false, 4, 1, 16)
+      }
     } else if (wide) {
-      if (rg <= 2) DS_FAST2(16, true, 2, 2, 8) else DS_FAST2(16, true, 4, 4, 4)
+      if (rg <= 1) DS_FAST2(16, true, 1, 1, 8) else if (rg <= 2) DS_FAST2(16, true, 2, 2, 8) else DS_FAST2(16, true, 4, 4, 4)
     } else {
-      if (rg <= 2) DS_FAST2(16, false, 2, 1, 8) else DS_FAST2(16, false, 4, 1, 8)
+      if (rg <= 1) DS_FAST2(16, false, 1, 1, 16) else if (rg <= 2) DS_FAST2(16, false, 2, 1, 16) else DS_FAST2(16, false, 4, 1, 8)
     }
 #undef DS_FAST2
 #undef DS_FAST3
