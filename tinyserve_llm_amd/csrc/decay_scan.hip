@@ -139,7 +139,7 @@ decay_scan_kernel(float* __restrict__ out, const float* __restrict__ q, int64_t 
 
 // The same walk where everything comes in whole 16-byte pieces (dim and vdim multiples of four up to 256 dimensions,
 // rows and places 16-byte aligned). A column's rows are dealt out in fours to GROUPS shares (4 for heads of less than 64
-// dimensions, else 16): share g takes the fours g, g + GROUPS, ... in ascending order, and the shares' sums meet in a
+// dimensions, 16 up to 127, else 32): share g takes the fours g, g + GROUPS, ... in ascending order, and the shares' sums meet in a
 // tree (neighbours first). Narrow form: a share is a lane, 64 / GROUPS columns a wave, the tree is the wave's exchanges.
 // Wide form (steps of few tokens a request): a lane keeps a whole column and all its shares' sums, 64 columns a wave, so
 // that the state's rows are read and written whole cache lines at a time; the tree is the same, so is every bit of the
@@ -345,8 +345,8 @@ extern "C" int ts_decay_scan(float* out, const float* q, int64_t q_stride, const
   const bool pieces = dim <= 256 && dim % 4 == 0 && vdim % 4 == 0 && ((q_stride | k_stride | v_stride | w_stride | state_stride) & 3) == 0 &&
                       (((uintptr_t)q | (uintptr_t)k | (uintptr_t)v | (uintptr_t)w) & 15) == 0;
   if (pieces) {
-    const int groups = dim < 64 ? 4 : 16;                   // (by the head's size alone: both forms then sum in one order)
-    if (!wide && groups == 16) waves = 4;                   // (4 columns a wave: a workgroup's waves share what is staged)
+    const int groups = dim < 64 ? 4 : dim < 128 ? 16 : 32;  // (by the head's size alone: both forms then sum in one order)
+    if (!wide && groups >= 16) waves = 4;                   // (4 or 2 columns a wave: a workgroup's waves share what is staged)
     const int wc = wide ? 64 : TS_WAVE / groups;
     const int cols = waves * wc;
     const int slices = (vdim + cols - 1) / cols;
@@ -372,10 +372,16 @@ extern "C" int ts_decay_scan(float* out, const float* q, int64_t q_stride, const
       } else {
         if (rg == 1) DS_FAST2(4, false, 1, 1, 16) else if (rg == 2) DS_FAST2(4, false, 2, 1, 16) else DS_FAST2(4, false, 4, 1, 16)
       }
+    } else if (groups == 16) {
+      if (wide) {
+        if (rg <= 1) DS_FAST2(16, true, 1, 1, 8) else DS_FAST2(16, true, 2, 2, 8)
+      } else {
+        if (rg <= 1) DS_FAST2(16, false, 1, 1, 16) else DS_FAST2(16, false, 2, 1, 16)
+      }
     } else if (wide) {
-      if (rg <= 1) DS_FAST2(16, true, 1, 1, 8) else if (rg <= 2) DS_FAST2(16, true, 2, 2, 8) else DS_FAST2(16, true, 4, 4, 4)
+      if (rg <= 1) DS_FAST2(32, true, 1, 2, 8) else DS_FAST2(32, true, 2, 4, 4)
     } else {
-      if (rg <= 1) DS_FAST2(16, false, 1, 1, 16) else if (rg <= 2) DS_FAST2(16, false, 2, 1, 16) else DS_FAST2(16, false, 4, 1, 8)
+      if (rg <= 1) DS_FAST2(32, false, 1, 1, 16) else DS_FAST2(32, false, 2, 1, 8)
     }
 #undef DS_FAST2
 #undef DS_FAST3
